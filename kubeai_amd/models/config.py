@@ -81,6 +81,8 @@ class ModelArchConfig:
             return dulotar_arch_config(cfg)
         if cfg.get("architecture") == "Nugopel":
             return nugopel_arch_config(cfg)
+        if cfg.get("architecture") == "Vekusun":
+            return vekusun_arch_config(cfg)
         hidden = cfg["hidden_size"]
         n_heads = cfg["num_attention_heads"]
         arch = (cfg.get("architectures") or ["LlamaForCausalLM"])[0]
@@ -196,6 +198,13 @@ class HybridSpec:
     norm_eps: float
     embedding_scale: float
     canon_taps: int  # taps of the per-layer input convolution (0 = none)
+    # multiplier on every layer's summed sublayer outputs
+    residual_mult: float = 1.0
+    # logits <- cap * tanh(logits / cap); 0 = none
+    logit_softcap: float = 0.0
+    # (start, stop, times): layers start..stop-1 run `times` times in a row
+    # with the same weights, every pass with cache and state of its own
+    loop: tuple = (0, 0, 1)
 
 
 def dulotar_arch_config(cfg: dict) -> ModelArchConfig:
@@ -257,6 +266,46 @@ def nugopel_arch_config(cfg: dict) -> ModelArchConfig:
             norm_eps=float(cfg["norm"]["eps"]),
             embedding_scale=1.0,
             canon_taps=0,
+        ),
+    )
+
+
+def vekusun_arch_config(cfg: dict) -> ModelArchConfig:
+    """Vekusun config.json -> arch config: the list of layers (mixer type, the
+    mixer's sizes and constants, the feed-forward), the looped span, the
+    residual multiplier, the logit cap and the norm epsilon, all as the file
+    gives them."""
+    layers = [
+        HybridLayerSpec(type=L["type"], mixer=L["mixer"], mlp=L.get("mlp"), weights_of=i)
+        for i, L in enumerate(cfg["layers"])
+    ]
+    loop = cfg.get("loop") or {}
+    start, stop = int(loop.get("start", 0)), int(loop.get("stop", 0))
+    times = int(loop.get("times", 1))
+    if not (0 <= start <= stop <= len(layers)) or times < 1:
+        raise ValueError(f"loop {loop!r} does not fit {len(layers)} layers")
+    if start == stop:
+        start, stop, times = 0, 0, 1
+    return ModelArchConfig(
+        architecture="vekusun",
+        vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]),
+        num_hidden_layers=len(layers),
+        intermediate_size=0,
+        num_attention_heads=0,
+        num_key_value_heads=0,
+        head_dim=0,
+        max_position_embeddings=1 << 30,  # positions are computed, not tabulated
+        bos_token_id=-1,
+        eos_token_id=-1,  # the design defines no end token
+        hybrid=HybridSpec(
+            layers=layers,
+            norm_eps=float(cfg["norm"]["eps"]),
+            embedding_scale=1.0,
+            canon_taps=0,
+            residual_mult=float(cfg.get("residual_mult", 1.0)),
+            logit_softcap=float(cfg.get("logit_softcap") or 0.0),
+            loop=(start, stop, times),
         ),
     )
 
@@ -729,6 +778,47 @@ def nugopel_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 
     })
 
 
+def vekusun_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
+                   kv_rank: int = 256, rot_dim: int = 64, experts: int = 8,
+                   top: int = 2, loop_times: int = 1) -> ModelArchConfig:
+    """A Vekusun stack of the given size with random-init weights: the layer
+    pattern (latent attention with a query latent and sinks + dense
+    feed-forward, latent attention with a rotated key part and head gates +
+    routed experts, gated delta rule + dense feed-forward, latent attention +
+    routed experts) repeats to the requested depth. The feed-forward work per
+    token is that of a dense 3.5 x width gated layer in either kind; with
+    loop_times > 1 the first two layers run that many times."""
+    heads = max(1, width // head_dim)
+    ff_dense = max(16, int(5.25 * width) // 16 * 16)        # two matrices
+    ff_exp = max(16, int(3.5 * width / top) // 16 * 16)     # three matrices, top experts
+    dense = {"kind": "dense", "ff": ff_dense}
+    moe = {"kind": "moe", "expert": {"ff": ff_exp},
+           "router": {"experts": experts, "top": top}}
+    lat1 = {"heads": heads, "dim": head_dim, "vdim": head_dim, "kv_rank": kv_rank,
+            "q_rank": max(64, width // 2), "scale": head_dim ** -0.5}
+    lat2 = {"heads": heads, "dim": head_dim, "rot_dim": rot_dim, "vdim": head_dim,
+            "kv_rank": kv_rank, "scale": (head_dim + rot_dim) ** -0.5,
+            "rot": {"base": 10000.0, "dims": rot_dim,
+                    "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0,
+                                "slow": 1.0}}}
+    delta = {"heads": heads, "kv_heads": max(1, heads // 2), "dim": head_dim,
+             "vdim": head_dim, "conv": 4}
+    pattern = [
+        {"type": "latent_attention", "mixer": lat1, "mlp": dense},
+        {"type": "latent_attention_2", "mixer": lat2, "mlp": moe},
+        {"type": "delta", "mixer": delta, "mlp": dense},
+        {"type": "latent_attention", "mixer": lat1, "mlp": moe},
+    ]
+    cfg = {
+        "architecture": "Vekusun", "vocab": vocab, "width": width,
+        "norm": {"eps": 1e-5}, "residual_mult": 1.0, "logit_softcap": 30.0,
+        "layers": [dict(pattern[i % 4]) for i in range(layers)],
+    }
+    if loop_times > 1:
+        cfg["loop"] = {"start": 0, "stop": min(2, layers), "times": loop_times}
+    return vekusun_arch_config(cfg)
+
+
 def dulotar_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
                    chunk: int = 1024, ff_mult: int = 4) -> ModelArchConfig:
     """A Dulotar stack of the given size with random-init weights: the
@@ -766,6 +856,11 @@ PRESETS.update({
     "nugopel-1k": nugopel_preset(1024, 12),
     "nugopel-2k": nugopel_preset(2048, 12),
     "nugopel-4k": nugopel_preset(4096, 6),
+    "vekusun-tiny": vekusun_preset(128, 4, vocab=512, head_dim=32, kv_rank=48,
+                                   rot_dim=16, experts=4, top=2, loop_times=2),
+    "vekusun-1k": vekusun_preset(1024, 12),
+    "vekusun-2k": vekusun_preset(2048, 12),
+    "vekusun-4k": vekusun_preset(4096, 6),
     "dulotar-tiny": dulotar_preset(128, 3, vocab=512, head_dim=32, chunk=64),
     "dulotar-1k": dulotar_preset(1024, 12),
     "dulotar-2k": dulotar_preset(2048, 12),

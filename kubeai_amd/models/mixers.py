@@ -41,10 +41,11 @@ class CausalConvTails(nn.Module):
     """Depthwise causal convolution over time whose last taps-1 inputs are
     sequence state (the layer-input convolution and the q/k/v convolutions)."""
 
-    def __init__(self, channels: int, taps: int, residual: bool):
+    def __init__(self, channels: int, taps: int, residual: bool, act: str = "none"):
         super().__init__()
         self.taps = taps
         self.residual = residual
+        self.act = act
         self.weight = _f32(channels, taps)
         nn.init.normal_(self.weight, std=0.3)
         self.channels = channels
@@ -53,7 +54,7 @@ class CausalConvTails(nn.Module):
         return (self.taps - 1, self.channels)
 
     def forward(self, x, fb, tails):
-        return sops.causal_conv(x, self.weight, tails, fb.seq, self.residual)
+        return sops.causal_conv(x, self.weight, tails, fb.seq, self.residual, self.act)
 
 
 class MinGRUMixer(nn.Module):
@@ -313,6 +314,8 @@ class SinkWindowAttention(nn.Module):
         self.register_buffer(
             "inv_freq", scaled_rotary_frequencies(rot_dims, rot_base, rot_scaling),
             persistent=False)
+        # the sink of this mixer is a key of score 0 for every head
+        self.sink_scores = _f32(heads) if self.sink else None
 
     def state_spec(self):
         return {}
@@ -333,29 +336,85 @@ class SinkWindowAttention(nn.Module):
                                         fb.slot_mapping)
         out = torch.empty((T, self.heads, self.vdim), dtype=h.dtype, device=h.device)
         sops.masked_paged_attention(q, k_cache, v_cache, fb.seq, self.scale, out,
-                                    window=self.window, sink=self.sink)
+                                    window=self.window, sink=self.sink_scores)
         return self.o_proj(out.view(T, self.heads * self.vdim))
+
+
+def ramped_rotary_frequencies(dims: int, base: float, scaling: dict | None):
+    """fp32 [dims/2] rotary frequencies f_i = base^(-2i/dims) and the factor
+    that multiplies cos and sin. With scaling = {factor, original, fast,
+    slow}, pair i is interpolated between its own frequency and f_i / factor
+    by a ramp over the pair index: the ramp runs from the pair that turns
+    `fast` times within `original` positions to the one that turns `slow`
+    times, d(t) = dims ln(original / (2 pi t)) / (2 ln base),
+    lo = max(floor d(fast), 0), hi = min(ceil d(slow), dims - 1),
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
+    f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i); the multiplier is
+    0.1 ln(factor) + 1 (1 without scaling)."""
+    import math
+
+    f = [float(base) ** (-2.0 * i / dims) for i in range(int(dims) // 2)]
+    mult = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def d(turns):
+            return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+        lo = max(math.floor(d(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(d(float(scaling["slow"]))), dims - 1)
+        for i, fi in enumerate(f):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            f[i] = fi / factor * ramp + fi * (1.0 - ramp)
+        mult = 0.1 * math.log(factor) + 1.0
+    return torch.tensor(f, dtype=torch.float32), mult
 
 
 class LatentAttention(nn.Module):
     """Causal attention whose keys and values are per-head up-projections of
     one low-rank latent per token; only the (RMS-normed) latent is cached,
-    as a one-head paged cache. No positions enter the scores. The heads'
-    concatenated output is gated by sigmoid of a projection of the input.
+    as a one-head paged cache. Options, each a constructor argument:
+
+      q_rank    queries go through a latent of their own: an RMS-normed
+                down-projection followed by an up-projection (0 = one matrix)
+      rot_dim   every query head has rot_dim more dimensions that are rotated
+                by position, against one rotated key part shared by all heads
+                and cached behind the latent (0 = no positions enter)
+      sink      a learned score per head that joins the softmax denominator
+                without a value
+      gate      "channel": every output channel times sigmoid of a projection
+                of the input; "head": one such gate per head; None
 
     The kernel attends in latent space: the key up-projection is folded into
     the query (q_h W_uk_h, one product per head), scores and the weighted sum
-    run against the cached latents, and the value up-projection is applied
-    to the result. With own_latent=False the layer has no down-projection and
-    reads the cache of another layer (bound by the model)."""
+    run against the cached rows (the rotated parts just extend the dot
+    product), and the value up-projection is applied to the attended latent.
+    With own_latent=False the layer has no down-projection and reads the
+    cache of another layer (bound by the model)."""
 
     def __init__(self, width, heads, dim, vdim, kv_rank, scale, own_latent=True,
-                 eps=1e-5):
+                 eps=1e-5, q_rank=0, rot_dim=0, rot_base=10000.0, rot_scaling=None,
+                 sink=False, gate="channel"):
         super().__init__()
         self.heads, self.dim, self.vdim, self.rank = heads, dim, vdim, kv_rank
         self.scale, self.own_latent, self.eps = float(scale), bool(own_latent), eps
-        self.sizes = (heads * dim, heads * vdim, kv_rank if own_latent else 0)
-        self.in_proj = Proj(width, sum(self.sizes))  # q | gate | latent
+        self.q_rank, self.rot_dim, self.gate = int(q_rank or 0), int(rot_dim or 0), gate
+        if gate not in ("channel", "head", None):
+            raise ValueError(f"unknown gate {gate!r}")
+        if self.rot_dim % 2:
+            raise ValueError("rot_dim must be even")
+        if self.rot_dim and not own_latent:
+            raise ValueError("a borrowed latent carries no rotated key part")
+        qd = dim + self.rot_dim
+        n_q = self.q_rank if self.q_rank else heads * qd
+        n_g = {"channel": heads * vdim, "head": heads, None: 0}[gate]
+        self.sizes = (n_q, n_g, kv_rank + self.rot_dim if own_latent else 0)
+        self.in_proj = Proj(width, sum(self.sizes))  # q (or its latent) | gate | latent
+        self.q_norm = self.q_up = None
+        if self.q_rank:
+            self.q_norm = _f32(self.q_rank)
+            nn.init.ones_(self.q_norm)
+            self.q_up = Proj(self.q_rank, heads * qd)
         self.latent_norm = None
         if own_latent:
             self.latent_norm = _f32(kv_rank)
@@ -367,29 +426,108 @@ class LatentAttention(nn.Module):
         self.uv = nn.Parameter(torch.empty(heads, vdim, kv_rank), requires_grad=False)
         nn.init.normal_(self.uk_r, std=kv_rank ** -0.5)
         nn.init.normal_(self.uv, std=kv_rank ** -0.5)
+        self.sink_scores = _f32(heads) if sink else None
+        freqs, self.rot_mult = ramped_rotary_frequencies(
+            max(self.rot_dim, 1), rot_base, rot_scaling)
+        self.register_buffer("inv_freq", freqs[: self.rot_dim // 2], persistent=False)
         self.o_proj = Proj(heads * vdim, width)
 
     def state_spec(self):
         return {}
 
     def kv_spec(self):
-        # one "head" of kv_rank dims; keys and values are the same rows
-        return (1, self.rank, 0) if self.own_latent else None
+        # one "head" of kv_rank (+ rot_dim) dims; keys and values are the same
+        # rows, the values their first kv_rank columns
+        return (1, self.rank + self.rot_dim, 0) if self.own_latent else None
 
     def forward(self, h, fb, state, kv_cache):
         T = h.shape[0]
-        H, D, Dv, R = self.heads, self.dim, self.vdim, self.rank
+        H, D, Dv, R, r = self.heads, self.dim, self.vdim, self.rank, self.rot_dim
         nq, ng, _ = self.sizes
         proj = self.in_proj(h)
         c_cache = kv_cache[0]
-        if self.own_latent:
+        if self.q_rank:
+            q = self.q_up(sops.rmsnorm_rows(proj[:, :nq], self.q_norm, self.eps))
+        else:
+            q = proj[:, :nq]
+        q = q.unflatten(-1, (H, D + r))
+        ql = torch.empty((T, H, R + r), dtype=h.dtype, device=h.device)
+        if self.own_latent and r:
+            sops.latent_rope_to_cache(proj[:, nq + ng :], self.latent_norm, self.eps,
+                                      q[..., D:], ql[..., R:], fb.positions,
+                                      self.inv_freq, self.rot_mult, c_cache,
+                                      fb.slot_mapping)
+        elif self.own_latent:
             sops.rmsnorm_to_cache(proj[:, nq + ng :], self.latent_norm, self.eps,
                                   c_cache, fb.slot_mapping)
-        ql = sops.head_linear(proj[:, :nq].unflatten(-1, (H, D)), self.uk_r)  # [T, H, R]
+        sops.head_linear(q[..., :D], self.uk_r, out=ql[..., :R])  # [T, H, R]
         lat = torch.empty((T, H, R), dtype=h.dtype, device=h.device)
-        sops.masked_paged_attention(ql, c_cache, c_cache, fb.seq, self.scale, lat)
-        o = sops.head_linear(lat, self.uv, gate=proj[:, nq : nq + ng])  # [T, H, Dv]
+        sops.masked_paged_attention(ql, c_cache, c_cache[..., :R] if r else c_cache,
+                                    fb.seq, self.scale, lat, sink=self.sink_scores)
+        o = sops.head_linear(lat, self.uv,
+                             gate=proj[:, nq : nq + ng] if ng else None)  # [T, H, Dv]
         return self.o_proj(o.view(T, H * Dv))
+
+
+class GatedDeltaMixer(nn.Module):
+    """Gated delta rule: a matrix state per head that decays by a
+    data-dependent factor and is corrected towards the current value along
+    the current key (S <- g S; S += k (beta (v - S^T k))^T; o = S^T q).
+    q and k have kv_heads heads shared by groups of value heads; q, k and v
+    pass a short causal convolution with silu; q and k are unit vectors per
+    head (q times dim^-1/2). The read-out is RMS-normed per head (one weight
+    vector shared by the heads) and gated by silu of a projection."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, conv_taps, eps):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.heads, self.kv_heads, self.dim, self.vdim, self.eps = heads, kv_heads, dim, vdim, eps
+        nqk, nv = kv_heads * dim, heads * vdim
+        self.sizes = (nqk, nqk, nv, nv, heads, heads)  # q | k | v | gate | beta | decay
+        self.in_proj = Proj(width, sum(self.sizes))
+        self.conv = CausalConvTails(2 * nqk + nv, conv_taps, residual=False, act="silu")
+        self.a_log = _f32(heads)
+        self.dt_bias = _f32(heads)
+        self.norm = _f32(nv)  # the per-head weight, repeated for every head
+        nn.init.ones_(self.norm)
+        self.o_proj = Proj(nv, width)
+
+    def state_spec(self):
+        return {"conv": self.conv.state_shape(),
+                "s": (self.heads, self.dim, self.vdim)}
+
+    def kv_spec(self):
+        return None
+
+    def forward(self, h, fb, state, kv_cache):
+        T = h.shape[0]
+        H, G, D, Dv = self.heads, self.kv_heads, self.dim, self.vdim
+        nqk, nv = G * D, H * Dv
+        proj = self.in_proj(h)
+        qkv = self.conv(proj[:, : 2 * nqk + nv], fb, state["conv"])
+        at = 2 * nqk + 2 * nv
+        o = sops.gated_delta_scan(
+            qkv[:, :nqk].unflatten(-1, (G, D)), qkv[:, nqk : 2 * nqk].unflatten(-1, (G, D)),
+            qkv[:, 2 * nqk :].unflatten(-1, (H, Dv)), proj[:, at : at + H],
+            proj[:, at + H : at + 2 * H], self.a_log, self.dt_bias,
+            state["s"], fb.seq)
+        y = torch.empty((T, nv), dtype=h.dtype, device=h.device)
+        sops.gated_rmsnorm(o.view(T, nv), self.norm, proj[:, 2 * nqk + nv : at], H,
+                           "silu", self.eps, y)
+        return self.o_proj(y)
+
+
+class GeluMLP(nn.Module):
+    """Dense feed-forward: down(gelu(up(h))), the exact (erf) GELU."""
+
+    def __init__(self, width: int, ff: int):
+        super().__init__()
+        self.up = Proj(width, ff)
+        self.down = Proj(ff, width)
+
+    def forward(self, h):
+        return self.down(sops.gelu(self.up(h)))
 
 
 class RoutedSquaredReluMoE(nn.Module):
@@ -446,4 +584,58 @@ class RoutedSquaredReluMoE(nn.Module):
             u = F.linear(h, self.up.weight[E * ff :])
             y = F.linear(sops.relu_squared(u), self.down.weight[:, E * ff :])
             out.add_(y)
+        return out
+
+
+class RoutedGatedMoE(nn.Module):
+    """Mixture of gated experts (down(silu(gate h) * (up h)), no biases).
+    Routing: fp32 logits, scores = softmax over all experts; the `top`
+    experts with the largest score + correction (a per-expert bias that only
+    steers the choice) are used, weighted by their scores as they are.
+
+    Expert e's gate and up matrices are rows [e*2ff, e*2ff + ff) and
+    [e*2ff + ff, (e+1)*2ff) of one stacked matrix, all down-projections one
+    [width, E*ff]. Small steps (decode) run two GEMMs over every expert with
+    the routing weight (0 for experts a token did not choose) folded into the
+    activation, so the weighted sum happens inside the second GEMM's fp32
+    accumulation and the step has no data-dependent shapes. Large steps
+    gather each expert's tokens and run its slice."""
+
+    DENSE_MAX_TOKENS = 256
+
+    def __init__(self, width, experts, top, ff, correction=True):
+        super().__init__()
+        self.experts, self.top, self.ff = experts, top, ff
+        self.router = nn.Parameter(torch.empty(experts, width, dtype=torch.float32),
+                                   requires_grad=False)
+        nn.init.normal_(self.router, std=width ** -0.5)
+        self.correction = _f32(experts) if correction else None
+        self.gate_up = Proj(width, experts * 2 * ff)
+        self.down = Proj(experts * ff, width)
+
+    def forward(self, h):
+        T = h.shape[0]
+        E, ff = self.experts, self.ff
+        logits = F.linear(h.float(), self.router)
+        dense, w, idx = sops.router_scores_topk(logits, self.top, self.correction)
+        if T <= self.DENSE_MAX_TOKENS:
+            return self.down(sops.silu_mul_weighted(self.gate_up(h), dense, ff))
+        out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
+        flat = idx.flatten().long()
+        order = torch.argsort(flat, stable=True)
+        counts = torch.bincount(flat, minlength=E).tolist()
+        tok = order // self.top
+        wrow = w.flatten()[order].unsqueeze(1)
+        s = 0
+        for e in range(E):
+            n = counts[e]
+            if n == 0:
+                continue
+            rows = tok[s : s + n]
+            gu = F.linear(h.index_select(0, rows),
+                          self.gate_up.weight[e * 2 * ff : (e + 1) * 2 * ff])
+            a = sops.silu_mul_weighted(gu, wrow[s : s + n], ff)
+            y = F.linear(a, self.down.weight[:, e * ff : (e + 1) * ff])
+            out.index_add_(0, rows, y.float())
+            s += n
         return out

@@ -21,11 +21,18 @@ def _nugopel():
     return NugopelForCausalLM
 
 
+def _vekusun():
+    from .vekusun import VekusunForCausalLM
+
+    return VekusunForCausalLM
+
+
 MODEL_REGISTRY = {
     "llama": _llama,
     "mixtral": _llama,
     "dulotar": _dulotar,
     "nugopel": _nugopel,
+    "vekusun": _vekusun,
 }
 
 
@@ -45,6 +52,7 @@ MODEL_EXTENSIONS = {
     "mixtral": ("_C",),
     "dulotar": ("_C_seq",),
     "nugopel": ("_C_seq",),
+    "vekusun": ("_C_seq",),
 }
 
 

@@ -148,12 +148,80 @@ def relu_squared(x):
     return (r * r).to(x.dtype)
 
 
+def gelu(x):
+    """Exact GELU, x * Phi(x) = x/2 (1 + erf(x / sqrt 2)), elementwise (fp32
+    inside)."""
+    if x.is_cuda:
+        _require_ext()
+        out = torch.empty_like(x)
+        _C.gelu(out, x)
+        return out
+    xf = x.float()
+    return (0.5 * xf * (1.0 + torch.erf(xf * 0.7071067811865476))).to(x.dtype)
+
+
+def rmsnorm_rows(x, weight, eps: float):
+    """x / sqrt(mean(x^2) + eps) * weight per row, fp32 inside. x [T, C] may
+    be a strided column view; returns a dense [T, C] of x's dtype."""
+    if x.is_cuda:
+        _require_ext()
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _C.rmsnorm_rows(out, x, weight, eps)
+        return out
+    xf = x.float()
+    return (xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps) * weight).to(x.dtype)
+
+
+def scaled_add_rmsnorm(residual, a, a_scale, b, b_scale, mult: float, extra,
+                       extra_row, weight, eps: float, out_dtype):
+    """Residual update of a layer whose sublayers read one norm and are
+    summed, fused with the next norm:
+
+        residual (fp32, in place) += mult * (a * a_scale + b * b_scale)
+        residual += extra + extra_row
+        returns residual / sqrt(mean(residual^2) + eps) * weight  (out_dtype)
+
+    a, b: branch outputs [T, C] (serving dtype or fp32), either may be None;
+    a_scale, b_scale: fp32 [C] per-channel scales (None = 1); extra: fp32
+    [T, C] or None; extra_row: fp32 [C] or None."""
+    if residual.is_cuda:
+        _require_ext()
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+        _C.scaled_add_rmsnorm(out, residual, a, a_scale, b, b_scale, mult, extra,
+                              extra_row, weight, eps)
+        return out
+    br = None
+    for t, sc in ((a, a_scale), (b, b_scale)):
+        if t is None:
+            continue
+        t = t.float() if sc is None else t.float() * sc
+        br = t if br is None else br + t
+    if br is not None:
+        residual.add_(br * mult)
+    if extra is not None:
+        residual.add_(extra)
+    if extra_row is not None:
+        residual.add_(extra_row)
+    r = torch.rsqrt((residual * residual).mean(-1, keepdim=True) + eps)
+    return (residual * r * weight).to(out_dtype)
+
+
+def tanh_cap(x, cap: float):
+    """cap * tanh(x / cap) on an fp32 tensor, in place."""
+    if x.is_cuda:
+        _require_ext()
+        _C.tanh_cap(x, cap)
+        return x
+    return x.copy_(cap * torch.tanh(x / cap))
+
+
 # ---------------------------------------------------------------------------
 # short causal convolutions with carried tails
 # ---------------------------------------------------------------------------
 
-def causal_conv(x, w, tails, meta: SeqMeta, residual: bool):
-    """Depthwise causal convolution over time inside every run.
+def causal_conv(x, w, tails, meta: SeqMeta, residual: bool, act: str = "none"):
+    """Depthwise causal convolution over time inside every run, followed by
+    an optional activation (act: "none" or "silu", applied to the sum).
 
     x [T, C] (row-strided view allowed); w fp32 [C, taps]:
     y_t = sum_j w[:, j] * x_(t - taps + 1 + j)  (+ x_t if residual).
@@ -166,7 +234,8 @@ def causal_conv(x, w, tails, meta: SeqMeta, residual: bool):
         _require_ext()
         y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         _C.causal_conv(y, x, w, tails, meta.start_loc, meta.slots,
-                       meta.token_seq, meta.positions, residual)
+                       meta.token_seq, meta.positions, residual,
+                       {"none": 0, "silu": 1}[act])
         return y
     y = torch.empty(x.shape, dtype=x.dtype)
     C = x.shape[1]
@@ -182,6 +251,10 @@ def causal_conv(x, w, tails, meta: SeqMeta, residual: bool):
         acc = xs.clone() if residual else torch.zeros_like(xs)
         for j in range(taps):
             acc += w[:, j] * full[j : j + n]
+        if act == "silu":
+            acc = acc * torch.sigmoid(acc)
+        elif act != "none":
+            raise ValueError(f"unknown activation {act!r}")
         y[s0 : s0 + n] = acc.to(x.dtype)
         if slot >= 0:
             tails[slot] = full[n : n + taps - 1]
@@ -284,6 +357,51 @@ def linear_attn_scan(q, k, v, decay, bonus, state, meta: SeqMeta, *,
             else:
                 S = decay.view(H, 1, 1) * S + kv
                 o[s0 + t] = torch.einsum("hkv,hk->hv", S, qs[t])
+        if slot >= 0:
+            state[slot] = S
+    return o
+
+
+def gated_delta_scan(q, k, v, beta_pre, decay_pre, a_log, dt_bias, state,
+                     meta: SeqMeta, norm_eps: float = 1e-6):
+    """Gated delta rule, per head a matrix state S [D, Dv] (fp32):
+
+        q <- q / sqrt(|q|^2 + norm_eps) * D^(-1/2),  k <- k / sqrt(|k|^2 + norm_eps)
+        beta = sigmoid(beta_pre),  g = exp(-exp(a_log_h) softplus(decay_pre + dt_bias_h))
+        S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+
+    so a token's read-out sees its own write. q, k [T, G, D] with H a
+    multiple of G (head h uses q/k head h // (H/G)), v [T, H, Dv], beta_pre
+    and decay_pre [T, H] (strided column views allowed), a_log and dt_bias
+    fp32 [H], state fp32 [slots, H, D, Dv]. Everything but the loads is fp32.
+    Returns o fp32 [T, H, Dv]."""
+    T, G, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    if q.is_cuda:
+        _require_ext()
+        o = torch.empty((T, H, Dv), dtype=torch.float32, device=q.device)
+        _C.gated_delta_scan(o, q, k, v, beta_pre, decay_pre, a_log, dt_bias,
+                            state, meta.start_loc, meta.slots, meta.positions,
+                            norm_eps, meta.max_len)
+        return o
+    o = torch.empty((T, H, Dv), dtype=torch.float32)
+    rep = H // G
+    for s0, n, slot, p0 in meta.runs():
+        qs, ks, vs = (a[s0 : s0 + n].float() for a in (q, k, v))
+        qs = qs * torch.rsqrt((qs * qs).sum(-1, keepdim=True) + norm_eps) * D ** -0.5
+        ks = ks * torch.rsqrt((ks * ks).sum(-1, keepdim=True) + norm_eps)
+        qs = qs.repeat_interleave(rep, dim=1)
+        ks = ks.repeat_interleave(rep, dim=1)
+        beta = torch.sigmoid(beta_pre[s0 : s0 + n].float())
+        g = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(
+            decay_pre[s0 : s0 + n].float() + dt_bias))
+        S = (state[slot].clone() if (slot >= 0 and p0 > 0)
+             else torch.zeros(H, D, Dv))
+        for t in range(n):
+            S = S * g[t].view(H, 1, 1)
+            u = beta[t].view(H, 1) * (vs[t] - torch.einsum("hkv,hk->hv", S, ks[t]))
+            S = S + ks[t].unsqueeze(-1) * u.unsqueeze(-2)
+            o[s0 + t] = torch.einsum("hkv,hk->hv", S, qs[t])
         if slot >= 0:
             state[slot] = S
     return o
@@ -410,6 +528,48 @@ def rmsnorm_to_cache(x, weight, eps: float, cache, slot_mapping):
     flat[slot_mapping[ok].long()] = y[ok].to(cache.dtype)
 
 
+def latent_rope_to_cache(x, weight, eps: float, q_rot, q_out, positions,
+                         inv_freq, rot_mult: float, cache, slot_mapping):
+    """Cache row of a latent-attention layer with a shared rotated key part.
+
+    x [T, R + r] (strided rows fine): the first R = len(weight) columns are
+    RMS-normed (times weight) into the cache row's first R columns; the last
+    r = 2 len(inv_freq) columns are rotated and written behind them. The
+    rotation pairs dimension 2i with 2i+1: (u, w) -> (u cos a - w sin a,
+    w cos a + u sin a) * rot_mult, a = position * inv_freq[i], fp32. The same
+    rotation is applied to q_rot [T, H, r] (a strided slice of the query
+    heads), written to q_out [T, H, r] (a strided slice of the folded query).
+    r may be 0 (q_rot/q_out None): only the norm runs. cache
+    [blocks, 1, block, R + r]; rows with slot < 0 are not written."""
+    R = weight.numel()
+    half = inv_freq.numel()
+    if x.is_cuda:
+        _require_ext()
+        _C.latent_rope_to_cache(cache, x, weight, eps, q_rot, q_out, positions,
+                                inv_freq, rot_mult, slot_mapping)
+        return
+    xf = x.float()
+    c = xf[:, :R]
+    row = [c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * weight]
+    if half:
+        a = positions.float().unsqueeze(-1) * inv_freq
+        cs, sn = torch.cos(a) * rot_mult, torch.sin(a) * rot_mult
+
+        def rot(t, cs, sn):
+            u, w = t[..., 0::2], t[..., 1::2]
+            o = torch.empty_like(t)
+            o[..., 0::2] = u * cs - w * sn
+            o[..., 1::2] = w * cs + u * sn
+            return o
+
+        row.append(rot(xf[:, R:], cs, sn))
+        q_out.copy_(rot(q_rot.float(), cs.unsqueeze(1), sn.unsqueeze(1)).to(q_out.dtype))
+    y = torch.cat(row, dim=-1)
+    ok = slot_mapping >= 0
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping[ok].long()] = y[ok].to(cache.dtype)
+
+
 def sigmoid_gate(x, gate, out=None):
     """x * sigmoid(gate), elementwise; gate may be a strided column view."""
     if out is None:
@@ -422,21 +582,26 @@ def sigmoid_gate(x, gate, out=None):
     return out
 
 
-def head_linear(x, w, gate=None):
-    """y[t, h, :] = w[h] @ x[t, h, :], times sigmoid(gate[t, h, :]) if a gate
-    is given. x [T, H, A] (a view with strided rows is fine), w [H, B, A],
-    gate [T, H*B] (strided rows fine) -> y [T, H, B], fp32 accumulation."""
+def head_linear(x, w, gate=None, out=None):
+    """y[t, h, :] = w[h] @ x[t, h, :], times sigmoid of a gate if one is
+    given: gate [T, H*B] gates every output channel, gate [T, H] a whole
+    head. x [T, H, A] and out [T, H, B] may be views whose token and head
+    strides are larger than their sizes (a slice of every head of a wider
+    buffer); w [H, B, A]; gate rows may be strided. fp32 accumulation."""
     T, H, _ = x.shape
     B = w.shape[1]
+    if out is None:
+        out = torch.empty((T, H, B), dtype=x.dtype, device=x.device)
     if x.is_cuda:
         _require_ext()
-        y = torch.empty((T, H, B), dtype=x.dtype, device=x.device)
-        _C.head_linear(y, x, w, gate)
-        return y
+        _C.head_linear(out, x, w, gate)
+        return out
     y = torch.einsum("tha,hba->thb", x.float(), w.float())
     if gate is not None:
-        y = y * torch.sigmoid(gate.float()).reshape(T, H, B)
-    return y.to(x.dtype).contiguous()
+        g = torch.sigmoid(gate.float())
+        y = y * (g.reshape(T, H, 1) if gate.shape[1] == H and B != 1 else g.reshape(T, H, B))
+    out.copy_(y.to(x.dtype))
+    return out
 
 
 # ---------------------------------------------------------------------------
@@ -480,6 +645,46 @@ def relu_squared_weighted(u, w, group: int):
     return r.to(u.dtype)
 
 
+def router_scores_topk(logits, top: int, bias=None):
+    """Routing by scores: s = softmax(logits) over all experts (fp32); the
+    `top` experts with the largest s + bias are chosen (equal values: lower
+    index first; bias fp32 [E] or None), and their weights are their scores
+    s themselves, not renormalised. Returns (dense [T, E] with the weights at
+    the chosen experts' columns, weights [T, top], index int32 [T, top])."""
+    T, E = logits.shape
+    if logits.is_cuda:
+        _require_ext()
+        dense = torch.empty((T, E), dtype=torch.float32, device=logits.device)
+        w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+        idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        _C.router_scores_topk(logits.contiguous(), bias, dense, w, idx)
+        return dense, w, idx
+    s = torch.softmax(logits.float(), dim=-1)
+    choice = s if bias is None else s + bias
+    idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    w = torch.gather(s, 1, idx)
+    dense = torch.zeros((T, E), dtype=torch.float32)
+    dense.scatter_(1, idx, w)
+    return dense, w, idx.to(torch.int32)
+
+
+def silu_mul_weighted(gu, w, group: int):
+    """Gated expert activation with the routing weight folded in. gu
+    [T, n * 2 * group] holds, per expert e, `group` gate columns followed by
+    `group` up columns; out[t, e * group + c] = silu(gate) * up * w[t, e].
+    w fp32 [T, n] (a strided column view is fine)."""
+    T, C2 = gu.shape
+    n = C2 // (2 * group)
+    if gu.is_cuda:
+        _require_ext()
+        out = torch.empty((T, n * group), dtype=gu.dtype, device=gu.device)
+        _C.silu_mul_weighted(out, gu, w, group)
+        return out
+    g = gu.float().view(T, n, 2, group)
+    a = g[:, :, 0] * torch.sigmoid(g[:, :, 0]) * g[:, :, 1] * w.unsqueeze(-1)
+    return a.reshape(T, n * group).to(gu.dtype)
+
+
 # ---------------------------------------------------------------------------
 # masked paged attention (decode tokens and prompt portions alike)
 # ---------------------------------------------------------------------------
@@ -487,16 +692,23 @@ def relu_squared_weighted(u, w, group: int):
 def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
                            out, *, softcap: float = 0.0, chunk: int = 0,
                            window: int = 0, out_scale: float = 1.0,
-                           sink: bool = False):
+                           sink: Optional[torch.Tensor] = None):
     """Softmax attention of every packed token over its own sequence's cached
     keys. The token at position i sees j <= i with, when chunk > 0,
     floor(j / chunk) == floor(i / chunk) (position-aligned chunks) and, when
     window > 0, j > i - window. Scores are (q . k) * scale, then
-    softcap * tanh(score / softcap) if softcap > 0; all in fp32. With sink,
-    the softmax has one more key of score 0 that carries no value (the
-    denominator grows by exp(0)).
-    q [T, H, D] (strided ok), caches [blocks, G, block, D | Dv];
-    out [T, H, Dv] may be a strided view; out = attention * out_scale."""
+    softcap * tanh(score / softcap) if softcap > 0; all in fp32. With sink
+    (fp32 [H]), the softmax of head h has one more key whose score is
+    sink[h] as it stands (not scaled, not capped) and that carries no value:
+    the denominator grows by exp(sink[h]).
+    q [T, H, D] (strided ok), caches [blocks, G, block, D | Dv]; v_cache may
+    be the leading Dv columns of the key rows (a view of k_cache);
+    out [T, H, Dv] may be a strided view; out = attention * out_scale.
+    sink=True stands for a score of 0 on every head."""
+    if sink is True:
+        sink = torch.zeros(q.shape[1], dtype=torch.float32, device=q.device)
+    elif sink is False:
+        sink = None
     if q.is_cuda:
         _require_ext()
         _C.masked_paged_attention(out, q, k_cache, v_cache, meta.block_tables,
@@ -535,10 +747,11 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
         if window > 0:
             vis &= j.view(1, -1) > pos.view(-1, 1) - window
         s = s.masked_fill(~vis.unsqueeze(0), float("-inf"))
-        if sink:
-            s = torch.cat([s, torch.zeros_like(s[..., :1])], dim=-1)
+        if sink is not None:
+            s = torch.cat(
+                [s, sink.float().view(H, 1, 1).expand(H, s.shape[1], 1)], dim=-1)
         p = torch.softmax(s, dim=-1)
-        if sink:
+        if sink is not None:
             p = p[..., :-1]
         o = torch.einsum("htl,lhd->thd", p, vs) * out_scale
         out[s0 : s0 + n] = o.to(out.dtype)

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
     const T* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ token_seq,
     const int* __restrict__ positions, float scale, float softcap, int chunk,
-    int window, float out_scale, int sink, int H, int G, int D, int Dv, int bs) {
+    int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G, int D, int Dv, int bs) {
   constexpr int N = Vec16<T>::N;
   const int lpr = kVec ? Dv / N : 1;          // lanes per value row
   const int ngrp = kVec ? WAVE / lpr : 1;     // key groups of a wave
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
       }
       sc = dot * scale;
       if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
-      vb = rowi * Dv;
+      vb = rowi * v_rs;
     }
     const float m_new = fmaxf(m, wave_max(sc));  // finite: lane 0's key is visible
     const float p = j <= pos ? expf(sc - m_new) : 0.f;
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
     wsc[w] = mw == -INFINITY ? 0.f : expf(mw - mx);  // a wave may have had no tile
     lsum += stat[2 * w + 1] * wsc[w];
   }
-  if (sink) lsum += expf(-mx);
+  if (sink != nullptr) lsum += expf(sink[h] - mx);
   const float inv = out_scale / lsum;
   for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
     float a = 0.f;
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
     const bf16raw* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ start_loc,
     const int* __restrict__ positions, int tiles_per_run, float scale,
-    float softcap, int chunk, int window, float out_scale, int sink, int H, int G,
+    float softcap, int chunk, int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G,
     int D, int Dv, int bs) {
   const int s = blockIdx.x / tiles_per_run, tile = blockIdx.x % tiles_per_run;
   const int h = blockIdx.y, g = h / (H / G);
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
       sc[i] = vis[i] ? x : -INFINITY;
       mt = fmaxf(mt, sc[i]);
       const int jv = min(j, pos_max);
-      vrow[i] = (((int64_t)bt[jv / bs] * G + g) * bs + jv % bs) * Dv;
+      vrow[i] = (((int64_t)bt[jv / bs] * G + g) * bs + jv % bs) * v_rs;
     }
     mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE));
     mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE));
@@ -389,7 +389,7 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
   }
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
-  if (sink) l += expf(-m);
+  if (sink != nullptr) l += expf(sink[h] - m);
   if (q_ok) {
     const float inv = out_scale / l;
     bf16raw* op = out + (size_t)tq * out_stride + h * Dv + grp * 4;
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(512) void masked_prefill_mfma_shared_kernel(
     const bf16raw* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ start_loc,
     const int* __restrict__ positions, int tiles_per_run, float scale,
-    float softcap, int chunk, int window, float out_scale, int sink, int H, int G,
+    float softcap, int chunk, int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G,
     int D, int Dv, int bs, int HW, int QW) {
   extern __shared__ __attribute__((aligned(16))) bf16raw lds[];
   constexpr int kKVec = kKT * kMaxDSteps * 16 / 8 / 256;   // per thread, 256 threads
@@ -528,7 +528,7 @@ __global__ __launch_bounds__(512) void masked_prefill_mfma_shared_kernel(
       if (c < vcpr) {
         const int j = min(j0 + row, bpos_max);
         vreg[i] = *(const uint4*)(v_cache +
-            (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * Dv + c * 8);
+            (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * v_rs + c * 8);
       }
     }
   };
@@ -637,7 +637,7 @@ __global__ __launch_bounds__(512) void masked_prefill_mfma_shared_kernel(
   }
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
-  if (sink) l += __builtin_amdgcn_exp2f(-m);
+  if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[h] * kLog2e - m);
   if (q_ok) {
     const float inv = out_scale / l;
     bf16raw* op = out + (size_t)tq * out_stride + h * Dv + grp * 4;
@@ -671,7 +671,7 @@ __global__ __launch_bounds__(kDW * WAVE) void masked_decode_mfma_kernel(
     const bf16raw* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ token_seq,
     const int* __restrict__ positions, float scale, float softcap, int chunk,
-    int window, float out_scale, int sink, int H, int G, int D, int Dv, int bs,
+    int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G, int D, int Dv, int bs,
     int n_split, float* __restrict__ part_o, float* __restrict__ part_ml) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
@@ -710,7 +710,7 @@ __global__ __launch_bounds__(kDW * WAVE) void masked_decode_mfma_kernel(
       const int row = v % kKT, c = v / kKT;
       const int j = min(j0 + row, pos);
       const uint4 x = *(const uint4*)(v_cache +
-          (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * Dv + c * 8);
+          (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * v_rs + c * 8);
       const uint32_t wv[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -804,7 +804,7 @@ __global__ __launch_bounds__(kDW * WAVE) void masked_decode_mfma_kernel(
       a += co[((size_t)w * 16 + hh) * Dv + d] * wsc;
     }
     if (n_split == 1) {
-      if (sink) lsum += __builtin_amdgcn_exp2f(-mx);
+      if (sink != nullptr) lsum += __builtin_amdgcn_exp2f(sink[h0 + hh] * kLog2e - mx);
       stf(out + (size_t)t * out_stride + (h0 + hh) * Dv + d, a * out_scale / lsum);
     } else {
       // partial result of this split: [t][head][split] -> (max, sum), values
@@ -823,7 +823,7 @@ __global__ void decode_split_join_kernel(bf16raw* __restrict__ out, int64_t out_
                                          const float* __restrict__ part_o,
                                          const float* __restrict__ part_ml, int H,
                                          int Dv, int n_split, float out_scale,
-                                         int sink) {
+                                         const float* __restrict__ sink) {
   const int t = blockIdx.x, h = blockIdx.y;
   const size_t row0 = ((size_t)t * H + h) * n_split;
   float mx = -INFINITY;
@@ -837,7 +837,7 @@ __global__ void decode_split_join_kernel(bf16raw* __restrict__ out, int64_t out_
       lsum += part_ml[(row0 + s) * 2 + 1] * w;
       a += part_o[(row0 + s) * Dv + d] * w;
     }
-    if (sink) lsum += __builtin_amdgcn_exp2f(-mx);
+    if (sink != nullptr) lsum += __builtin_amdgcn_exp2f(sink[h] * kLog2e - mx);
     stf(out + (size_t)t * out_stride + h * Dv + d, a * out_scale / lsum);
   }
 }
@@ -940,17 +940,29 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                             torch::Tensor token_seq, torch::Tensor positions,
                             int64_t max_len, double scale, double softcap,
                             int64_t chunk, int64_t window, double out_scale,
-                            bool sink) {
+                            c10::optional<torch::Tensor> sink_scores) {
   check_i32(start_loc, "start_loc");
   check_i32(block_tables, "block_tables");
   check_i32(token_seq, "token_seq");
   check_i32(positions, "positions");
   TORCH_CHECK(dense_heads3(q) && dense_heads3(out));
   const int T = q.size(0), H = q.size(1), D = q.size(2);
-  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
-              k_cache.dim() == 4 && v_cache.dim() == 4);
+  TORCH_CHECK(k_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4);
   const int G = k_cache.size(1), bs = k_cache.size(2), Dv = v_cache.size(3);
   TORCH_CHECK(k_cache.size(3) == D && v_cache.size(1) == G && v_cache.size(2) == bs);
+  // value rows may be the leading columns of wider rows (of the key rows,
+  // when a layer caches one row per token that serves as both)
+  const int64_t v_rs = v_cache.stride(2);
+  TORCH_CHECK(v_cache.is_cuda() && (Dv == 1 || v_cache.stride(3) == 1) && v_rs >= Dv &&
+              v_cache.stride(1) == (int64_t)bs * v_rs &&
+              v_cache.stride(0) == (int64_t)G * bs * v_rs,
+              "value cache rows must be evenly spaced");
+  const float* sink = nullptr;
+  if (sink_scores.has_value()) {
+    check_f32(*sink_scores, "sink_scores");
+    TORCH_CHECK(sink_scores->numel() == H, "one sink score per head");
+    sink = (const float*)sink_scores->data_ptr();
+  }
   TORCH_CHECK(G > 0 && H % G == 0 && H <= 65535);
   TORCH_CHECK(out.size(0) == T && out.size(1) == H && out.size(2) == Dv);
   TORCH_CHECK(Dv <= kMaxDvPerLane * WAVE, "value size too large");
@@ -966,7 +978,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
     return ((size_t)t.data_ptr()) % 8 == 0 && t.stride(0) % 4 == 0;
   };
   if (q.scalar_type() == torch::kBFloat16 && max_len > 1 && D % 16 == 0 &&
-      Dv % 16 == 0 && D <= 512 && Dv <= 512 && al8(q) && al8(out)) {
+      Dv % 16 == 0 && D <= 512 && Dv <= 512 && al8(q) && al8(out) && v_rs % 8 == 0) {
     // prompt portions: matrix-core kernel over 16-query tiles of every run
     const int tiles = (int)((max_len + 15) / 16);
     auto launch = [&](auto kern) {
@@ -979,7 +991,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
                          (const int*)positions.data_ptr(), tiles, (float)scale,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                         (int)sink, H, G, D, Dv, bs);
+                         sink, v_rs, H, G, D, Dv, bs);
     };
     const size_t lds_shared =
         (size_t)2 * (kKT * (D + kKPad) + Dv * (kKT + kVPad)) * sizeof(bf16raw);
@@ -1007,7 +1019,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
                          (const int*)positions.data_ptr(), btiles, (float)scale,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                         (int)sink, H, G, D, Dv, bs, HW, QW);
+                         sink, v_rs, H, G, D, Dv, bs, HW, QW);
       };
       if (D % 32 == 0) launch_shared(masked_prefill_mfma_shared_kernel<8, 16, true>);
       else launch_shared(masked_prefill_mfma_shared_kernel<8, 16, false>);
@@ -1022,7 +1034,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
   // worth it when many heads share a row (measured: 16 heads on one latent
   // 60 -> 28 us per call, groups of 4 no faster than the generic kernel)
   if (q.scalar_type() == torch::kBFloat16 && max_len == 1 && H / G >= 8 && D % 16 == 0 &&
-      Dv % 16 == 0 && D <= 128 && Dv <= 128 && al8(q) &&
+      Dv % 16 == 0 && D <= 128 && Dv <= 128 && al8(q) && v_rs % 8 == 0 &&
       ((size_t)k_cache.data_ptr()) % 16 == 0 && ((size_t)v_cache.data_ptr()) % 16 == 0) {
     // decode tokens: the heads of a key/value group are the rows of a tile
     const int rep = H / G, zb = (rep + 15) / 16;
@@ -1050,7 +1062,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                        (const int*)block_tables.data_ptr(), (int)block_tables.size(1),
                        (const int*)token_seq.data_ptr(), (const int*)positions.data_ptr(),
                        (float)scale, (float)softcap, (int)chunk, (int)window,
-                       (float)out_scale, (int)sink, H, G, D, Dv, bs, n_split,
+                       (float)out_scale, sink, v_rs, H, G, D, Dv, bs, n_split,
                        n_split > 1 ? (float*)part_o.data_ptr() : nullptr,
                        n_split > 1 ? (float*)part_ml.data_ptr() : nullptr);
     if (n_split > 1) {
@@ -1059,7 +1071,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (bf16raw*)out.data_ptr(), out.stride(0),
                          (const float*)part_o.data_ptr(),
                          (const float*)part_ml.data_ptr(), H, (int)Dv, n_split,
-                         (float)out_scale, (int)sink);
+                         (float)out_scale, sink);
     }
     SEQ_CHECK_LAUNCH();
     return;
@@ -1069,7 +1081,8 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
     // 16-byte row loads need whole vectors per key / value row and at most
     // one wave of lanes per value row
     const bool vec = D % N == 0 && Dv % N == 0 && Dv / N <= WAVE && Dv >= N &&
-                     N <= kMaxDvPerLane;
+                     N <= kMaxDvPerLane && v_rs % N == 0 &&
+                     ((size_t)v_cache.data_ptr()) % 16 == 0;
     const int ngrp = vec ? WAVE / (Dv / N) : 1;
     const size_t lds = (size_t)(3 * WAVE * kDecWaves + 2 * kDecWaves +
                                 ((D + 3) & ~3) + kDecWaves * ngrp * Dv) * 4;
@@ -1084,7 +1097,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (int)block_tables.size(1), (const int*)token_seq.data_ptr(),
                          (const int*)positions.data_ptr(), (float)scale,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                         (int)sink, H, G, D, Dv, bs);
+                         sink, v_rs, H, G, D, Dv, bs);
     };
     if (vec) launch(masked_paged_attention_kernel<act_t, true>);
     else launch(masked_paged_attention_kernel<act_t, false>);

@@ -11,7 +11,7 @@ void relu_squared(torch::Tensor out, torch::Tensor x);
 void causal_conv(torch::Tensor y, torch::Tensor x, torch::Tensor w,
                  torch::Tensor tails, torch::Tensor start_loc,
                  torch::Tensor slots, torch::Tensor token_seq,
-                 torch::Tensor positions, bool residual);
+                 torch::Tensor positions, bool residual, int64_t act);
 void token_shift_mix(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
                      torch::Tensor prev, torch::Tensor start_loc,
                      torch::Tensor slots, torch::Tensor token_seq,
@@ -35,7 +35,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                             torch::Tensor token_seq, torch::Tensor positions,
                             int64_t max_len, double scale, double softcap,
                             int64_t chunk, int64_t window, double out_scale,
-                            bool sink);
+                            c10::optional<torch::Tensor> sink_scores);
 void qknorm_rope_half_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
                                 c10::optional<torch::Tensor> q_weight,
                                 c10::optional<torch::Tensor> k_weight, double eps,
@@ -54,6 +54,32 @@ void router_topk(torch::Tensor logits, torch::Tensor dense, torch::Tensor weight
                  torch::Tensor index);
 void relu_squared_weighted(torch::Tensor out, torch::Tensor u, torch::Tensor w,
                            int64_t group);
+void scaled_add_rmsnorm(torch::Tensor out, torch::Tensor residual,
+                        c10::optional<torch::Tensor> a,
+                        c10::optional<torch::Tensor> a_scale,
+                        c10::optional<torch::Tensor> b,
+                        c10::optional<torch::Tensor> b_scale, double mult,
+                        c10::optional<torch::Tensor> extra,
+                        c10::optional<torch::Tensor> extra_row, torch::Tensor weight,
+                        double eps);
+void rmsnorm_rows(torch::Tensor out, torch::Tensor x, torch::Tensor weight, double eps);
+void gelu(torch::Tensor out, torch::Tensor x);
+void tanh_cap(torch::Tensor x, double cap);
+void latent_rope_to_cache(torch::Tensor cache, torch::Tensor x, torch::Tensor weight,
+                          double eps, c10::optional<torch::Tensor> q_rot,
+                          c10::optional<torch::Tensor> q_out, torch::Tensor positions,
+                          torch::Tensor inv_freq, double rot_mult,
+                          torch::Tensor slot_mapping);
+void router_scores_topk(torch::Tensor logits, c10::optional<torch::Tensor> bias,
+                        torch::Tensor dense, torch::Tensor weights,
+                        torch::Tensor index);
+void silu_mul_weighted(torch::Tensor out, torch::Tensor gu, torch::Tensor w,
+                       int64_t group);
+void gated_delta_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
+                      torch::Tensor v, torch::Tensor beta_pre, torch::Tensor decay_pre,
+                      torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor state,
+                      torch::Tensor start_loc, torch::Tensor slots,
+                      torch::Tensor positions, double norm_eps, int64_t max_len);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("add_layernorm", &add_layernorm, "fp32 residual add + LayerNorm");
@@ -78,4 +104,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("router_topk", &router_topk, "top-k routing with softmax over the chosen");
   m.def("relu_squared_weighted", &relu_squared_weighted,
         "relu(u)^2 times a per-row, per-group weight");
+  m.def("scaled_add_rmsnorm", &scaled_add_rmsnorm,
+        "fp32 residual += scaled sum of two branches (+ extras), then RMS norm");
+  m.def("rmsnorm_rows", &rmsnorm_rows, "row RMS norm of a strided view");
+  m.def("gelu", &gelu, "exact (erf) GELU");
+  m.def("tanh_cap", &tanh_cap, "cap * tanh(x / cap), in place, fp32");
+  m.def("latent_rope_to_cache", &latent_rope_to_cache,
+        "latent RMS norm + rotated shared key part into a paged cache, query rotation");
+  m.def("router_scores_topk", &router_scores_topk,
+        "softmax scores, biased top-k choice, unnormalised score weights");
+  m.def("silu_mul_weighted", &silu_mul_weighted,
+        "silu(gate) * up times a per-row, per-expert weight");
+  m.def("gated_delta_scan", &gated_delta_scan, "gated delta rule recurrence");
 }

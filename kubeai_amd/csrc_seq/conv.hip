@@ -10,13 +10,14 @@ constexpr int kMaxTail = 15;  // taps - 1
 // grid (T, ceil(C / 256)). Input d steps back comes from this run's tokens
 // when it lies inside the run, else from the carried tail; positions < 0
 // contribute zero. tails row i holds the input at position p0 - K1 + i.
+// act 1 applies silu to the sum.
 template <typename T>
 __global__ void causal_conv_kernel(
     T* __restrict__ y, const T* __restrict__ x, int64_t x_stride,
     const float* __restrict__ w, const float* __restrict__ tails,
     const int* __restrict__ start_loc, const int* __restrict__ slots,
     const int* __restrict__ token_seq, const int* __restrict__ positions,
-    int C, int taps, int residual) {
+    int C, int taps, int residual, int act) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
@@ -37,6 +38,7 @@ __global__ void causal_conv_kernel(
     }
     acc += w[(size_t)c * taps + j] * v;
   }
+  if (act == 1) acc = silu_f(acc);
   stf(y + (size_t)t * C + c, acc);
 }
 
@@ -104,8 +106,9 @@ static void launch_tail_update(torch::Tensor tails, torch::Tensor x,
 void causal_conv(torch::Tensor y, torch::Tensor x, torch::Tensor w,
                  torch::Tensor tails, torch::Tensor start_loc,
                  torch::Tensor slots, torch::Tensor token_seq,
-                 torch::Tensor positions, bool residual) {
+                 torch::Tensor positions, bool residual, int64_t act) {
   check_rows(x, "x");
+  TORCH_CHECK(act == 0 || act == 1, "act: 0 none, 1 silu");
   check_f32(w, "w");
   check_f32(tails, "tails");
   check_i32(start_loc, "start_loc");
@@ -128,7 +131,8 @@ void causal_conv(torch::Tensor y, torch::Tensor x, torch::Tensor w,
                        (const float*)w.data_ptr(), (const float*)tails.data_ptr(),
                        (const int*)start_loc.data_ptr(), (const int*)slots.data_ptr(),
                        (const int*)token_seq.data_ptr(),
-                       (const int*)positions.data_ptr(), C, taps, residual ? 1 : 0);
+                       (const int*)positions.data_ptr(), C, taps, residual ? 1 : 0,
+                       (int)act);
   });
   SEQ_CHECK_LAUNCH();
   launch_tail_update(tails, x, start_loc, slots, positions, C, taps - 1);

@@ -1,5 +1,7 @@
 // Per-head linear maps y[t, h, :] = W[h] x[t, h, :] (W[h] is [B, A], applied
-// like a Linear weight), with an optional sigmoid gate on the output. The
+// like a Linear weight), with an optional sigmoid gate on the output (one per
+// output channel, or one per head: gate_per_head). x and y may be slices of
+// the heads of wider buffers: heads are x_hs / y_hs elements apart. The
 // folded key / value up-projections of latent attention are such maps: the
 // heads are independent small matrices, so one launch covers all of them
 // and writes the token-major layout the attention kernels read.
@@ -19,10 +21,10 @@ constexpr int kHlWaves = 4;
 // channels of one token.
 template <int kSteps>
 __global__ __launch_bounds__(kHlWaves * WAVE) void head_linear_mfma_kernel(
-    bf16raw* __restrict__ y, int64_t y_stride, const bf16raw* __restrict__ x,
-    int64_t x_stride, const bf16raw* __restrict__ w,
-    const bf16raw* __restrict__ gate, int64_t gate_stride, int T, int H, int A,
-    int B) {
+    bf16raw* __restrict__ y, int64_t y_stride, int64_t y_hs,
+    const bf16raw* __restrict__ x, int64_t x_stride, int64_t x_hs,
+    const bf16raw* __restrict__ w, const bf16raw* __restrict__ gate,
+    int64_t gate_stride, int gate_per_head, int T, int H, int A, int B) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int col = lane & 15, grp = lane >> 4;
   const int t0 = (blockIdx.x * kHlWaves + wave) * 16;
@@ -32,7 +34,10 @@ __global__ __launch_bounds__(kHlWaves * WAVE) void head_linear_mfma_kernel(
   const bool t_ok = t0 + col < T;
   const int nks = A / 16;
   bf16x4 xf[kSteps];
-  const bf16raw* xr = x + (size_t)t * x_stride + (size_t)h * A + grp * 4;
+  const bf16raw* xr = x + (size_t)t * x_stride + (size_t)h * x_hs + grp * 4;
+  float hg = 1.f;
+  if (gate != nullptr && gate_per_head)
+    hg = sigmoid_f(bf16_to_f32(gate[(size_t)t * gate_stride + h]));
 #pragma unroll
   for (int ks = 0; ks < kSteps; ++ks)
     if (ks < nks) xf[ks] = *(const bf16x4*)(xr + ks * 16);
@@ -48,7 +53,9 @@ __global__ __launch_bounds__(kHlWaves * WAVE) void head_linear_mfma_kernel(
     if (t_ok) {
       const int c = b0 + grp * 4;
       float o[4] = {acc[0], acc[1], acc[2], acc[3]};
-      if (gate != nullptr) {
+      if (gate != nullptr && gate_per_head) {
+        o[0] *= hg; o[1] *= hg; o[2] *= hg; o[3] *= hg;
+      } else if (gate != nullptr) {
         const ushort4 g4 =
             *(const ushort4*)(gate + (size_t)t * gate_stride + (size_t)h * B + c);
         o[0] *= sigmoid_f(bf16_to_f32(g4.x));
@@ -61,7 +68,7 @@ __global__ __launch_bounds__(kHlWaves * WAVE) void head_linear_mfma_kernel(
       o4.y = f32_to_bf16(o[1]);
       o4.z = f32_to_bf16(o[2]);
       o4.w = f32_to_bf16(o[3]);
-      *(ushort4*)(y + (size_t)t * y_stride + (size_t)h * B + c) = o4;
+      *(ushort4*)(y + (size_t)t * y_stride + (size_t)h * y_hs + c) = o4;
     }
   }
 }
@@ -70,21 +77,27 @@ __global__ __launch_bounds__(kHlWaves * WAVE) void head_linear_mfma_kernel(
 // channel per thread at a time, fp32 accumulation.
 template <typename T_>
 __global__ __launch_bounds__(256) void head_linear_kernel(
-    T_* __restrict__ y, int64_t y_stride, const T_* __restrict__ x,
-    int64_t x_stride, const T_* __restrict__ w, const T_* __restrict__ gate,
-    int64_t gate_stride, int H, int A, int B) {
+    T_* __restrict__ y, int64_t y_stride, int64_t y_hs, const T_* __restrict__ x,
+    int64_t x_stride, int64_t x_hs, const T_* __restrict__ w,
+    const T_* __restrict__ gate, int64_t gate_stride, int gate_per_head, int H,
+    int A, int B) {
   extern __shared__ float xs[];
   const int t = blockIdx.x, h = blockIdx.y;
   for (int i = threadIdx.x; i < A; i += blockDim.x)
-    xs[i] = ldf(x + (size_t)t * x_stride + (size_t)h * A + i);
+    xs[i] = ldf(x + (size_t)t * x_stride + (size_t)h * x_hs + i);
   __syncthreads();
+  float hg = 1.f;
+  if (gate != nullptr && gate_per_head)
+    hg = sigmoid_f(ldf(gate + (size_t)t * gate_stride + h));
   for (int b = threadIdx.x; b < B; b += blockDim.x) {
     const T_* wr = w + ((size_t)h * B + b) * A;
     float acc = 0.f;
     for (int i = 0; i < A; ++i) acc += xs[i] * ldf(wr + i);
-    if (gate != nullptr)
+    if (gate != nullptr && gate_per_head)
+      acc *= hg;
+    else if (gate != nullptr)
       acc *= sigmoid_f(ldf(gate + (size_t)t * gate_stride + (size_t)h * B + b));
-    stf(y + (size_t)t * y_stride + (size_t)h * B + b, acc);
+    stf(y + (size_t)t * y_stride + (size_t)h * y_hs + b, acc);
   }
 }
 
@@ -98,18 +111,23 @@ void head_linear(torch::Tensor y, torch::Tensor x, torch::Tensor w,
   TORCH_CHECK(w.size(0) == H && w.size(2) == A && y.size(0) == T && y.size(1) == H &&
               y.size(2) == B);
   auto dense = [](const torch::Tensor& t) {
-    return (t.size(2) == 1 || t.stride(2) == 1) &&
-           (t.size(1) == 1 || t.stride(1) == t.size(2));
+    return (t.size(2) == 1 || t.stride(2) == 1) && t.stride(1) >= t.size(2) &&
+           t.stride(0) >= (t.size(1) - 1) * t.stride(1) + t.size(2);
   };
-  TORCH_CHECK(dense(x) && dense(y), "heads must be dense within a token's row");
+  TORCH_CHECK(dense(x) && dense(y),
+              "a head's channels must be dense and heads must not overlap");
+  const int64_t x_hs = x.stride(1), y_hs = y.stride(1);
   TORCH_CHECK(y.scalar_type() == x.scalar_type() && w.scalar_type() == x.scalar_type());
   TORCH_CHECK(H <= 65535);
   const void* gp = nullptr;
   int64_t gs = 0;
+  int gph = 0;
   if (gate.has_value()) {
     check_rows(*gate, "gate");
-    TORCH_CHECK(gate->size(0) == T && gate->size(1) == (int64_t)H * B &&
-                gate->scalar_type() == x.scalar_type());
+    TORCH_CHECK(gate->size(0) == T && gate->scalar_type() == x.scalar_type() &&
+                (gate->size(1) == (int64_t)H * B || gate->size(1) == H),
+                "gate must have one column per output channel or per head");
+    gph = gate->size(1) == H && B != 1;
     gp = gate->data_ptr();
     gs = gate->stride(0);
   }
@@ -119,14 +137,15 @@ void head_linear(torch::Tensor y, torch::Tensor x, torch::Tensor w,
   };
   if (x.scalar_type() == torch::kBFloat16 && A % 16 == 0 && B % 16 == 0 && A <= 512 &&
       al8(x.data_ptr(), x.stride(0)) && al8(y.data_ptr(), y.stride(0)) &&
-      al8(w.data_ptr(), 4) && (gp == nullptr || al8(gp, gs))) {
+      x_hs % 4 == 0 && y_hs % 4 == 0 && al8(w.data_ptr(), 4) &&
+      (gp == nullptr || gph || al8(gp, gs))) {
     const dim3 grid((T + 16 * kHlWaves - 1) / (16 * kHlWaves), H);
     auto launch = [&](auto kern) {
       hipLaunchKernelGGL(kern, grid, dim3(kHlWaves * WAVE), 0, SEQ_STREAM(),
-                         (bf16raw*)y.data_ptr(), y.stride(0),
-                         (const bf16raw*)x.data_ptr(), x.stride(0),
-                         (const bf16raw*)w.data_ptr(), (const bf16raw*)gp, gs, T, H, A,
-                         B);
+                         (bf16raw*)y.data_ptr(), y.stride(0), y_hs,
+                         (const bf16raw*)x.data_ptr(), x.stride(0), x_hs,
+                         (const bf16raw*)w.data_ptr(), (const bf16raw*)gp, gs, gph, T,
+                         H, A, B);
     };
     if (A <= 128) launch(head_linear_mfma_kernel<8>);
     else launch(head_linear_mfma_kernel<32>);
@@ -137,8 +156,8 @@ void head_linear(torch::Tensor y, torch::Tensor x, torch::Tensor w,
   SEQ_DISPATCH_ACT(x, {
     hipLaunchKernelGGL((head_linear_kernel<act_t>), dim3(T, H), dim3(256),
                        (size_t)A * 4, SEQ_STREAM(), (act_t*)y.data_ptr(), y.stride(0),
-                       (const act_t*)x.data_ptr(), x.stride(0),
-                       (const act_t*)w.data_ptr(), (const act_t*)gp, gs, H, A, B);
+                       y_hs, (const act_t*)x.data_ptr(), x.stride(0), x_hs,
+                       (const act_t*)w.data_ptr(), (const act_t*)gp, gs, gph, H, A, B);
   });
   SEQ_CHECK_LAUNCH();
 }

@@ -419,6 +419,7 @@ void gated_delta_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
         nseg = (int)((max_len + seg_len - 1) / seg_len);
       }
     }
+    if (nseg == 1) seg_len = (int)std::max<int64_t>(max_len, 1);  // one segment: the whole run
     torch::Tensor ws_p, ws_b, ws_s;
     if (nseg > 1) {
       ws_p = torch::empty({(int64_t)n_seq * nseg * H * D * D}, state.options());

@@ -446,6 +446,7 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
         nseg = (int)((max_len + seg_len - 1) / seg_len);
       }
     }
+    if (nseg == 1) seg_len = (int)std::max<int64_t>(max_len, 1);  // one segment: the whole run
     torch::Tensor wsB, wsW;
     if (nseg > 1) {
       wsB = torch::empty({(int64_t)n_seq * nseg * H * D * Dv}, state.options());

@@ -105,10 +105,10 @@ def rel_err(got, want):
     return np.abs(got - want).max(-1) / want.std()
 
 
-def check(got, want, dtype="float32"):
+def check(got, want, dtype="float32", loose=0.15):
     err = rel_err(got, want).max()
     # bf16: the widths here are tiny, so roundings do not average out
-    assert err < (2e-4 if dtype == "float32" else 0.15), f"relative error {err:.3g}"
+    assert err < (2e-4 if dtype == "float32" else loose), f"relative error {err:.3g}"
 
 
 def replay(eng, rid, toks, cuts):
@@ -465,16 +465,21 @@ SIXTEENS = config(
     width=64, vocab=80, loop=(0, 2, 2))
 
 
+# odd sizes: the generic kernels. With key sizes of 6 and 10 the reference ops
+# on the CPU land at 0.2 in bf16 for this model (0.06 for SIXTEENS).
+ODD = config([lat1(), delta(), lat2(mlp=moe(experts=3, top=3)), delta(mlp=None)],
+             loop=(1, 3, 2))
+
+
 @pytest.mark.parametrize("device", GPU)
-@pytest.mark.parametrize("name", ["mixed", "sixteens"])
+@pytest.mark.parametrize("name", ["odd_sizes", "sixteens"])
 def test_bfloat16_serving_precision(tmp_path, device, name):
-    cfg = {"mixed": config(MIXED["layers"][:3] + [delta(mlp=None)], loop=(1, 3, 2)),
-           "sixteens": SIXTEENS}[name]
+    cfg, loose = {"odd_sizes": (ODD, 0.4), "sixteens": (SIXTEENS, 0.15)}[name]
     d, W = model_dir(tmp_path, cfg, seed=9)
     toks = tokens(70, cfg["vocab"], 7)
     want = oracle.forward(cfg, W, toks)
-    check(replay(engine(d, device, "bfloat16"), "a", toks, [len(toks)]), want, "bfloat16")
-    check(replay(engine(d, device, "bfloat16"), "b", toks, [33, 2, 1]), want, "bfloat16")
+    check(replay(engine(d, device, "bfloat16"), "a", toks, [len(toks)]), want, "bfloat16", loose)
+    check(replay(engine(d, device, "bfloat16"), "b", toks, [33, 2, 1]), want, "bfloat16", loose)
     check(replay(engine(d, device, "float32"), "c", toks, [33, 2, 1]), want)
 
 
@@ -896,9 +901,35 @@ def test_kernel_attention_over_shared_rows_with_sinks(dtype, H, R, rot):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("n", [127, 128, 129, 200, 256, 257, 513])
+def test_kernel_scans_at_segment_borders(n):
+    """Run lengths around the sizes at which the scans start to cut a run
+    into parallel segments: the delta rule and the linear-attention scan."""
+    H, G, D, Dv = 2, 1, 16, 8
+    ins = _delta_inputs(n, H, G, D, Dv, n)
+    want = _delta_want(*ins)
+    pos = torch.arange(n, dtype=torch.int32).cuda()
+    meta = sops.SeqMeta.build([(n, 0)], pos, "cuda")
+    state = torch.zeros(1, H, D, Dv).cuda()
+    got = sops.gated_delta_scan(*(t.cuda() for t in ins), state, meta)
+    assert np.abs(npy(got) - want).max() < 5e-5
+    g = torch.Generator().manual_seed(n)
+    q, k = (torch.randn(n, H, D, generator=g) * 0.3 for _ in range(2))
+    v = torch.randn(n, H, Dv, generator=g)
+    decay = torch.tensor([0.9, 0.97])
+    res = []
+    for dev in ("cpu", "cuda"):
+        st = torch.zeros(1, H, D, Dv).to(dev)
+        m = sops.SeqMeta.build([(n, 0)], pos.to(dev), dev)
+        res.append(sops.linear_attn_scan(q.to(dev), k.to(dev), v.to(dev), decay.to(dev), None,
+                                         st, m).cpu())
+    assert float((res[0] - res[1]).abs().max()) < 1e-4
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 32, 16), (2, 1, 128, 40), (3, 3, 10, 6),
-                                      (8, 4, 64, 64)])
+                                      (8, 4, 64, 64), (2, 1, 64, 8)])
 def test_kernel_delta_scan(dtype, H, G, D, Dv):
     """Register-state and LDS-state kernels, plain and segment-parallel runs,
     inputs as strided column views of one projection, against the reference."""

@@ -1,9 +1,11 @@
-"""Prefill and decode throughput of a layer-list design (Dulotar, Nugopel)
-beside the closest homogeneous stack of equal width, depth and (about)
+"""Prefill and decode throughput of a layer-list design (Dulotar, Nugopel,
+Vekusun) beside the closest existing stack of equal width, depth and (about)
 parameter count, random weights, one GPU: a dense Llama for Dulotar, a
-Mixtral-style routed Llama (same number of experts and choices) for Nugopel.
+Mixtral-style routed Llama (same number of experts and choices) for Nugopel,
+and Nugopel itself (latent attention, routed experts) for Vekusun, whose
+feed-forward sizes are scaled so that the parameter counts agree.
 
-    python bench.py --compare-hybrid [--compare-design dulotar|nugopel]
+    python bench.py --compare-hybrid [--compare-design dulotar|nugopel|vekusun]
                     [--compare-sizes 1k,2k,4k]
 
 Prefill: one sequence's whole prompt as a single fixed step (both families
@@ -55,6 +57,24 @@ def _llama_like(width: int, layers: int, vocab: int, target_params: int,
         max_position_embeddings=16384, rope_theta=10000.0, eos_token_id=2,
         bos_token_id=1, num_local_experts=experts, num_experts_per_tok=top,
     )
+
+
+def _meta_params(arch: ModelArchConfig) -> int:
+    """Parameter count of an architecture without allocating it."""
+    from kubeai_amd.models.registry import model_class
+
+    return _params(model_class(arch.architecture)(arch, device="meta"))
+
+
+def _vekusun_sized_like(width: int, layers: int, target_params: int) -> ModelArchConfig:
+    """The Vekusun preset of this width and depth with its feed-forward sizes
+    scaled to the target parameter count (the count is linear in the scale)."""
+    from kubeai_amd.models.config import vekusun_preset
+
+    p1 = _meta_params(vekusun_preset(width, layers, ff_scale=1.0))
+    p2 = _meta_params(vekusun_preset(width, layers, ff_scale=2.0))
+    scale = 1.0 + (target_params - p1) / max(p2 - p1, 1)
+    return vekusun_preset(width, layers, ff_scale=max(scale, 0.1))
 
 
 def _engine(name: str, device: str, blocks: int, seqs: int, max_len: int):
@@ -120,11 +140,15 @@ def main(args) -> None:
     prefill_lens = [2048, 8192] if device == "cuda" else [64]
     batches = [(64, 1536), (8, 3584)] if device == "cuda" else [(2, 32)]
     design = getattr(args, "compare_design", None) or "dulotar"
-    if design not in ("dulotar", "nugopel"):
+    if design not in ("dulotar", "nugopel", "vekusun"):
         raise SystemExit(f"unknown design {design!r}")
     for key in sizes:
         width, layers = SIZES[key]
         name = f"{design}-{key}" if device == "cuda" else f"{design}-tiny"
+        if design == "vekusun" and device == "cuda":
+            name = f"vekusun-like-nugopel-{key}"
+            PRESETS[name] = _vekusun_sized_like(
+                width, layers, _meta_params(PRESETS[f"nugopel-{key}"]))
         arch = PRESETS[name]
         max_len = 8192 + 256
         blocks = (max(b * (c + 128) for b, c in batches) + max_len) // 16 + 64
@@ -134,7 +158,10 @@ def main(args) -> None:
         ref_name = f"llama-like-{key}"
         ref_fam = "llama"
         moe = arch.hybrid.layers[0].mlp if design == "nugopel" else None
-        if moe:
+        if design == "vekusun":
+            ref_fam = "nugopel"
+            ref_name = f"nugopel-{key}" if device == "cuda" else "nugopel-tiny"
+        elif moe:
             ref_fam = "mixtral"
             PRESETS[ref_name] = _llama_like(
                 arch.hidden_size, arch.num_hidden_layers, arch.vocab_size, n_params,

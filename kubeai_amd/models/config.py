@@ -780,17 +780,19 @@ def nugopel_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 
 
 def vekusun_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
                    kv_rank: int = 256, rot_dim: int = 64, experts: int = 8,
-                   top: int = 2, loop_times: int = 1) -> ModelArchConfig:
+                   top: int = 2, loop_times: int = 1,
+                   ff_scale: float = 1.0) -> ModelArchConfig:
     """A Vekusun stack of the given size with random-init weights: the layer
     pattern (latent attention with a query latent and sinks + dense
     feed-forward, latent attention with a rotated key part and head gates +
     routed experts, gated delta rule + dense feed-forward, latent attention +
     routed experts) repeats to the requested depth. The feed-forward work per
-    token is that of a dense 3.5 x width gated layer in either kind; with
-    loop_times > 1 the first two layers run that many times."""
+    token is that of a dense 3.5 x width gated layer in either kind (times
+    ff_scale, for matching another model's size); with loop_times > 1 the
+    first two layers run that many times."""
     heads = max(1, width // head_dim)
-    ff_dense = max(16, int(5.25 * width) // 16 * 16)        # two matrices
-    ff_exp = max(16, int(3.5 * width / top) // 16 * 16)     # three matrices, top experts
+    ff_dense = max(16, int(5.25 * ff_scale * width) // 16 * 16)     # two matrices
+    ff_exp = max(16, int(3.5 * ff_scale * width / top) // 16 * 16)  # three, top experts
     dense = {"kind": "dense", "ff": ff_dense}
     moe = {"kind": "moe", "expert": {"ff": ff_exp},
            "router": {"experts": experts, "top": top}}

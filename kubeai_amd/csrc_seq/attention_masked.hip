@@ -997,7 +997,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
         (size_t)2 * (kKT * (D + kKPad) + Dv * (kKT + kVPad)) * sizeof(bf16raw);
     const bool cache_al16 = ((size_t)k_cache.data_ptr()) % 16 == 0 &&
                             ((size_t)v_cache.data_ptr()) % 16 == 0;
-    if (D <= 128 && Dv <= 256 && lds_shared <= 64 * 1024 && cache_al16) {
+    if (D <= 256 && Dv <= 256 && lds_shared <= 64 * 1024 && cache_al16) {
       // tiles shared through LDS by up to 8 waves: heads of a group first,
       // then neighbouring query tiles
       const int rep = H / G;
@@ -1021,8 +1021,15 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
                          sink, v_rs, H, G, D, Dv, bs, HW, QW);
       };
-      if (D % 32 == 0) launch_shared(masked_prefill_mfma_shared_kernel<8, 16, true>);
-      else launch_shared(masked_prefill_mfma_shared_kernel<8, 16, false>);
+      // key sizes above 128 (a latent with a rotated part behind it) keep
+      // twice as many query fragments in registers
+      if (D <= 128) {
+        if (D % 32 == 0) launch_shared(masked_prefill_mfma_shared_kernel<8, 16, true>);
+        else launch_shared(masked_prefill_mfma_shared_kernel<8, 16, false>);
+      } else {
+        if (D % 32 == 0) launch_shared(masked_prefill_mfma_shared_kernel<16, 16, true>);
+        else launch_shared(masked_prefill_mfma_shared_kernel<16, 16, false>);
+      }
     } else if (D <= 128 && Dv <= 256) {
       launch(masked_prefill_mfma_kernel<8, 16>);
     } else {
@@ -1034,7 +1041,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
   // worth it when many heads share a row (measured: 16 heads on one latent
   // 60 -> 28 us per call, groups of 4 no faster than the generic kernel)
   if (q.scalar_type() == torch::kBFloat16 && max_len == 1 && H / G >= 8 && D % 16 == 0 &&
-      Dv % 16 == 0 && D <= 128 && Dv <= 128 && al8(q) && v_rs % 8 == 0 &&
+      Dv % 16 == 0 && D <= 256 && Dv <= 128 && al8(q) && v_rs % 8 == 0 &&
       ((size_t)k_cache.data_ptr()) % 16 == 0 && ((size_t)v_cache.data_ptr()) % 16 == 0) {
     // decode tokens: the heads of a key/value group are the rows of a tile
     const int rep = H / G, zb = (rep + 15) / 16;
@@ -1053,7 +1060,9 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
       part_o = torch::empty({(int64_t)T * H * n_split, Dv}, f32);
       part_ml = torch::empty({(int64_t)T * H * n_split, 2}, f32);
     }
-    hipLaunchKernelGGL((masked_decode_mfma_kernel<8, 8>), dim3(T, G, zb * n_split),
+    auto decode_kern = D <= 128 ? masked_decode_mfma_kernel<8, 8>
+                                : masked_decode_mfma_kernel<16, 8>;
+    hipLaunchKernelGGL(decode_kern, dim3(T, G, zb * n_split),
                        dim3(kDW * WAVE), stage > join ? stage : join, SEQ_STREAM(),
                        (bf16raw*)out.data_ptr(), out.stride(0),
                        (const bf16raw*)q.data_ptr(), q.stride(0),

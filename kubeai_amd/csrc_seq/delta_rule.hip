@@ -14,7 +14,8 @@
 // come out of the same recurrence: B by walking from zero, P by walking the
 // identity with zero values. Pass 1 (compose) walks every segment but the
 // last for P and B, pass 2 (fold) chains S_(i+1) = P_i S_i + B_i per column
-// block, pass 3 walks every segment from its incoming state and writes o.
+// block with P_i staged in LDS, pass 3 walks every segment from its incoming
+// state and writes o.
 #include "seq_common.h"
 
 namespace {
@@ -119,8 +120,8 @@ __global__ void gated_delta_scan_kernel(
 //   slot's state (first segment), or from seg_state[seg] (later ones);
 //   writes o, and the slot's state after the run's last segment.
 // mode 1 (compose): column blocks [0, D/16) are columns of the identity
-//   walked with zero values (-> seg_p), the rest value columns walked from
-//   zero (-> seg_b); the run's last segment is skipped.
+//   walked with zero values (-> seg_p, stored transposed), the rest value
+//   columns walked from zero (-> seg_b); the run's last segment is skipped.
 template <typename T, int kQ>
 __global__ __launch_bounds__(WAVE) void gated_delta_scan_reg_kernel(
     float* __restrict__ o, const T* __restrict__ q, int64_t q_stride,
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(WAVE) void gated_delta_scan_reg_kernel(
     if (ident) {
       float* pp = seg_p + sh * D * D;
 #pragma unroll
-      for (int i = 0; i < R; ++i) pp[(size_t)(r * R + i) * D + cb * 16 + c] = S[i];
+      for (int i = 0; i < R; ++i) pp[(size_t)(cb * 16 + c) * D + r * R + i] = S[i];  // P^T
     } else if (valid) {
       float* bp = seg_b + sh * D * Dv;
 #pragma unroll
@@ -299,58 +300,96 @@ __global__ __launch_bounds__(WAVE) void gated_delta_scan_reg_kernel(
   }
 }
 
-// Fold: grid (n_seq * H * ceil(Dv / 4)), one wave per 4 value columns of a
-// head. Lane (r, c), r = lane / 4, c = lane % 4, owns rows [r D/16,
-// (r+1) D/16) of column c. seg_state[0] is not written (the first segment
-// starts from the slot); seg_state[i + 1] = P_i seg_state[i] + B_i, the
-// column block passing through LDS between the steps.
+// Fold: grid (n_seq * H * column blocks), 256 threads. A block chains
+// seg_state[i + 1] = P_i seg_state[i] + B_i for CB = 4 * (256 / (D / 4))
+// value columns of one head (seg_state[0] is not written: the first segment
+// starts from the slot). Every thread owns a 4 x 4 tile of the column block.
+// P_i arrives transposed (seg_pt[k][i] = P_i[i][k]) and is staged in LDS as a
+// whole, fetched into registers while the previous step is computed; the
+// column block passes through LDS between the steps. Per contraction index a
+// thread reads one float4 of P^T and one of S for 16 products.
 template <int kD>
-__global__ __launch_bounds__(WAVE) void gated_delta_fold_kernel(
-    float* __restrict__ seg_state, const float* __restrict__ seg_p,
+__global__ __launch_bounds__(256) void gated_delta_fold_kernel(
+    float* __restrict__ seg_state, const float* __restrict__ seg_pt,
     const float* __restrict__ seg_b, const float* __restrict__ state,
     const int* __restrict__ start_loc, const int* __restrict__ slots,
-    const int* __restrict__ positions, int H, int Dv, int ncb4, int nseg,
+    const int* __restrict__ positions, int H, int Dv, int ncbk, int nseg,
     int seg_len) {
-  constexpr int RR = kD / 16;
-  const int cb = blockIdx.x % ncb4;
-  const int h = (blockIdx.x / ncb4) % H;
-  const int s = blockIdx.x / (ncb4 * H);
+  constexpr int RT = kD / 4;                       // row tiles
+  constexpr int CT = 256 / RT;                     // column tiles of a block
+  constexpr int CB = 4 * CT;                       // columns of a block
+  constexpr int PV = (kD * kD / 4 + 255) / 256;    // float4 of P per thread
+  extern __shared__ __attribute__((aligned(16))) float fold_sm[];
+  float* pt = fold_sm;            // [kD][kD]
+  float* sc = fold_sm + kD * kD;  // [kD][CB]
+  const int cb = blockIdx.x % ncbk;
+  const int h = (blockIdx.x / ncbk) % H;
+  const int s = blockIdx.x / (ncbk * H);
   const int r0 = start_loc[s], n = start_loc[s + 1] - r0, slot = slots[s];
   const int used = (n + seg_len - 1) / seg_len;  // segments this run has
-  if (used <= 1) return;
-  __shared__ float sc[kD * 4];
-  const int lane = threadIdx.x, r = lane >> 2, c = lane & 3;
-  const int j = cb * 4 + c;
-  const bool valid = j < Dv;
+  if (used <= 1) return;                         // the whole block
+  const int tid = threadIdx.x;
+  const int rt = tid % RT, ct = tid / RT;
+  const bool active = ct < CT;
+  const int i0 = rt * 4, c0 = ct * 4, j0 = cb * CB + c0;
   const bool carry = slot >= 0 && positions[r0] > 0;
   const float* sp = state + ((size_t)(slot < 0 ? 0 : slot) * H + h) * kD * Dv;
-  float S[RR];
+  float S[4][4];
 #pragma unroll
-  for (int i = 0; i < RR; ++i)
-    S[i] = (carry && valid) ? sp[(size_t)(r * RR + i) * Dv + j] : 0.f;
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      S[a][b] = (carry && active && j0 + b < Dv) ? sp[(size_t)(i0 + a) * Dv + j0 + b] : 0.f;
+  float4 pre[PV];
+  auto fetch = [&](int seg) {
+    const float4* src =
+        (const float4*)(seg_pt + (((size_t)s * nseg + seg) * H + h) * kD * kD);
+#pragma unroll
+    for (int v = 0; v < PV; ++v) {
+      const int idx = v * 256 + tid;
+      if (idx < kD * kD / 4) pre[v] = src[idx];
+    }
+  };
+  fetch(0);
   for (int seg = 0; seg + 1 < used; ++seg) {
     const size_t sh = ((size_t)s * nseg + seg) * H + h;
-    __syncthreads();
+    __syncthreads();  // the previous step's readers are done
 #pragma unroll
-    for (int i = 0; i < RR; ++i) sc[(r * RR + i) * 4 + c] = S[i];
-    __syncthreads();
-    const float* pp = seg_p + sh * kD * kD;
-    const float* bp = seg_b + sh * kD * Dv;
-#pragma unroll
-    for (int i = 0; i < RR; ++i) {
-      const float4* prow = (const float4*)(pp + (size_t)(r * RR + i) * kD);
-      float acc = valid ? bp[(size_t)(r * RR + i) * Dv + j] : 0.f;
-      for (int kk = 0; kk < kD / 4; ++kk) {
-        const float4 p = prow[kk];
-        acc += p.x * sc[(4 * kk) * 4 + c] + p.y * sc[(4 * kk + 1) * 4 + c] +
-               p.z * sc[(4 * kk + 2) * 4 + c] + p.w * sc[(4 * kk + 3) * 4 + c];
-      }
-      S[i] = acc;
+    for (int v = 0; v < PV; ++v) {
+      const int idx = v * 256 + tid;
+      if (idx < kD * kD / 4) ((float4*)pt)[idx] = pre[v];
     }
-    float* out = seg_state + (sh + H) * kD * Dv;  // segment seg + 1
-    if (valid) {
+    if (active) {
 #pragma unroll
-      for (int i = 0; i < RR; ++i) out[(size_t)(r * RR + i) * Dv + j] = S[i];
+      for (int a = 0; a < 4; ++a)
+        *(float4*)(sc + (i0 + a) * CB + c0) = make_float4(S[a][0], S[a][1], S[a][2], S[a][3]);
+    }
+    __syncthreads();
+    if (seg + 2 < used) fetch(seg + 1);
+    if (active) {
+      const float* bp = seg_b + sh * kD * Dv;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          S[a][b] = j0 + b < Dv ? bp[(size_t)(i0 + a) * Dv + j0 + b] : 0.f;
+#pragma unroll 4
+      for (int k = 0; k < kD; ++k) {
+        const float4 p = *(const float4*)(pt + k * kD + i0);
+        const float4 x = *(const float4*)(sc + k * CB + c0);
+        const float pa[4] = {p.x, p.y, p.z, p.w};
+        const float xa[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int b = 0; b < 4; ++b) S[a][b] += pa[a] * xa[b];
+      }
+      float* out = seg_state + (sh + H) * kD * Dv;  // segment seg + 1
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          if (j0 + b < Dv) out[(size_t)(i0 + a) * Dv + j0 + b] = S[a][b];
     }
   }
 }
@@ -447,13 +486,27 @@ void gated_delta_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                            nseg > 1 ? (const float*)ws_s.data_ptr() : nullptr);
       };
       auto launch_fold = [&](auto kern) {
-        const int ncb4 = (Dv + 3) / 4;
-        hipLaunchKernelGGL(kern, dim3(n_seq * H * ncb4), dim3(WAVE), 0, SEQ_STREAM(),
+        const int cbk = 4 * (256 / (D / 4));  // value columns of a fold block
+        const int ncbk = (Dv + cbk - 1) / cbk;
+        const size_t fold_lds = ((size_t)D * D + (size_t)D * cbk) * sizeof(float);
+        // raise the dynamic-LDS cap once per kernel, outside any capture
+        static thread_local const void* raised[8] = {};
+        if (fold_lds > 48 * 1024) {
+          bool seen = false;
+          for (auto p : raised) seen |= p == (const void*)kern;
+          if (!seen) {
+            hipFuncSetAttribute((const void*)kern,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            for (auto& p : raised)
+              if (p == nullptr) { p = (const void*)kern; break; }
+          }
+        }
+        hipLaunchKernelGGL(kern, dim3(n_seq * H * ncbk), dim3(256), fold_lds, SEQ_STREAM(),
                            (float*)ws_s.data_ptr(), (const float*)ws_p.data_ptr(),
                            (const float*)ws_b.data_ptr(), (const float*)state.data_ptr(),
                            (const int*)start_loc.data_ptr(),
                            (const int*)slots.data_ptr(),
-                           (const int*)positions.data_ptr(), H, Dv, ncb4, nseg, seg_len);
+                           (const int*)positions.data_ptr(), H, Dv, ncbk, nseg, seg_len);
       };
       auto launch = [&](auto kern) {
         if (nseg > 1) {

@@ -779,7 +779,7 @@ def nugopel_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 
 
 
 def vekusun_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
-                   kv_rank: int = 256, rot_dim: int = 64, experts: int = 8,
+                   kv_rank: int = 128, rot_dim: int = 64, experts: int = 8,
                    top: int = 2, loop_times: int = 1,
                    ff_scale: float = 1.0) -> ModelArchConfig:
     """A Vekusun stack of the given size with random-init weights: the layer

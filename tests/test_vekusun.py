@@ -873,7 +873,7 @@ def test_kernel_head_linear_on_slices_with_head_gate(dtype, T, H, A, B, pad):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,R,rot", [(4, 10, 6), (8, 64, 16), (16, 128, 64), (2, 32, 0),
-                                     (16, 48, 16)])
+                                     (16, 48, 16), (16, 96, 48), (8, 192, 64), (4, 256, 16)])
 def test_kernel_attention_over_shared_rows_with_sinks(dtype, H, R, rot):
     g = torch.Generator().manual_seed(H)
     bs, nblk = 16, 12
@@ -929,7 +929,8 @@ def test_kernel_scans_at_segment_borders(n):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 32, 16), (2, 1, 128, 40), (3, 3, 10, 6),
-                                      (8, 4, 64, 64), (2, 1, 64, 8)])
+                                      (8, 4, 64, 64), (2, 1, 64, 8), (2, 1, 48, 24),
+                                      (1, 1, 80, 100), (2, 2, 16, 300)])
 def test_kernel_delta_scan(dtype, H, G, D, Dv):
     """Register-state and LDS-state kernels, plain and segment-parallel runs,
     inputs as strided column views of one projection, against the reference."""

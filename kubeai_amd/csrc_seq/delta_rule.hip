@@ -24,8 +24,9 @@ constexpr int kTile = 16;  // tokens staged per barrier
 
 DEV_INLINE float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
-// Any size: grid (n_seq * H), block = Dv rounded up to a wave, the head's
-// state in LDS, thread j owns value column j.
+// Any size: grid (n_seq * H, column blocks), block = the block's columns
+// rounded up to a wave, that part of the head's state in LDS, thread j owns
+// value column c0 + j.
 template <typename T>
 __global__ void gated_delta_scan_kernel(
     float* __restrict__ o, const T* __restrict__ q, int64_t q_stride,
@@ -35,21 +36,25 @@ __global__ void gated_delta_scan_kernel(
     const float* __restrict__ a_log, const float* __restrict__ dt_bias,
     float* __restrict__ state, const int* __restrict__ start_loc,
     const int* __restrict__ slots, const int* __restrict__ positions, int H, int G,
-    int D, int Dv, float norm_eps) {
+    int D, int Dv, int CB, float norm_eps) {
   const int s = blockIdx.x / H, h = blockIdx.x % H;
   const int hk = h / (H / G);
   const int s0 = start_loc[s], s1 = start_loc[s + 1], slot = slots[s];
   if (s1 <= s0) return;
+  const int c0 = blockIdx.y * CB, nc = min(CB, Dv - c0);  // this block's columns
   extern __shared__ float sm[];
-  float* S = sm;                      // [D][Dv]
-  float* qs = S + (size_t)D * Dv;     // [tile][D]
+  float* S = sm;                      // [D][CB]
+  float* qs = S + (size_t)D * CB;     // [tile][D]
   float* ks = qs + kTile * D;         // [tile][D]
-  float* vs = ks + kTile * D;         // [tile][Dv]
-  float* gb = vs + kTile * Dv;        // [tile][2]: decay, beta
+  float* vs = ks + kTile * D;         // [tile][CB]
+  float* gb = vs + kTile * CB;        // [tile][2]: decay, beta
   const int tid = threadIdx.x, nthr = blockDim.x;
   const bool carry = slot >= 0 && positions[s0] > 0;
   float* sp = state + ((size_t)(slot < 0 ? 0 : slot) * H + h) * D * Dv;
-  for (int i = tid; i < D * Dv; i += nthr) S[i] = carry ? sp[i] : 0.f;
+  for (int i = tid; i < D * CB; i += nthr) {
+    const int r = i / CB, c = i % CB;
+    S[i] = (carry && c < nc) ? sp[(size_t)r * Dv + c0 + c] : 0.f;
+  }
   const float rate = -expf(a_log[h]), bias = dt_bias[h];
   const float qscale = 1.0f / sqrtf((float)D);
   for (int t0 = s0; t0 < s1; t0 += kTile) {
@@ -60,9 +65,9 @@ __global__ void gated_delta_scan_kernel(
       qs[i] = ldf(q + (size_t)(t0 + tt) * q_stride + hk * D + d);
       ks[i] = ldf(k + (size_t)(t0 + tt) * k_stride + hk * D + d);
     }
-    for (int i = tid; i < nt * Dv; i += nthr) {
-      const int tt = i / Dv, d = i % Dv;
-      vs[i] = ldf(v + (size_t)(t0 + tt) * v_stride + h * Dv + d);
+    for (int i = tid; i < nt * CB; i += nthr) {
+      const int tt = i / CB, d = i % CB;
+      vs[i] = d < nc ? ldf(v + (size_t)(t0 + tt) * v_stride + h * Dv + c0 + d) : 0.f;
     }
     __syncthreads();
     if (tid < nt) {
@@ -81,31 +86,34 @@ __global__ void gated_delta_scan_kernel(
       gb[2 * tid + 1] = sigmoid_f(ldf(beta_pre + (size_t)(t0 + tid) * b_stride + h));
     }
     __syncthreads();
-    if (tid < Dv) {
+    if (tid < nc) {
       for (int tt = 0; tt < nt; ++tt) {
         const float* qt = qs + tt * D;
         const float* kt = ks + tt * D;
         const float g = gb[2 * tt], beta = gb[2 * tt + 1];
         float dot = 0.f;
         for (int i = 0; i < D; ++i) {
-          const float st = g * S[i * Dv + tid];
-          S[i * Dv + tid] = st;
+          const float st = g * S[i * CB + tid];
+          S[i * CB + tid] = st;
           dot += st * kt[i];
         }
-        const float u = beta * (vs[tt * Dv + tid] - dot);
+        const float u = beta * (vs[tt * CB + tid] - dot);
         float acc = 0.f;
         for (int i = 0; i < D; ++i) {
-          const float st = S[i * Dv + tid] + kt[i] * u;
-          S[i * Dv + tid] = st;
+          const float st = S[i * CB + tid] + kt[i] * u;
+          S[i * CB + tid] = st;
           acc += qt[i] * st;
         }
-        o[((size_t)(t0 + tt) * H + h) * Dv + tid] = acc;
+        o[((size_t)(t0 + tt) * H + h) * Dv + c0 + tid] = acc;
       }
     }
   }
   __syncthreads();
   if (slot >= 0)
-    for (int i = tid; i < D * Dv; i += nthr) sp[i] = S[i];
+    for (int i = tid; i < D * CB; i += nthr) {
+      const int r = i / CB, c = i % CB;
+      if (c < nc) sp[(size_t)r * Dv + c0 + c] = S[i];
+    }
 }
 
 // Register-state form for key sizes D = 16 * kQ (<= 128). One wave per block
@@ -526,11 +534,17 @@ void gated_delta_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
     SEQ_CHECK_LAUNCH();
     return;
   }
-  const int threads = ((Dv + WAVE - 1) / WAVE) * WAVE;
-  TORCH_CHECK(threads <= 1024, "value size too large");
-  const size_t lds =
-      ((size_t)D * Dv + 2 * kTile * D + kTile * Dv + 2 * kTile) * sizeof(float);
-  TORCH_CHECK(lds <= 160 * 1024, "head state does not fit LDS");
+  // value columns per block: all of them if the state fits LDS, else fewer
+  // (columns are independent), in whole waves
+  auto lds_for = [&](int cb) {
+    return ((size_t)D * cb + 2 * kTile * D + (size_t)kTile * cb + 2 * kTile) * sizeof(float);
+  };
+  int CB = std::min(((Dv + WAVE - 1) / WAVE) * WAVE, 1024);
+  while (CB > WAVE && lds_for(CB) > 144 * 1024) CB -= WAVE;
+  const size_t lds = lds_for(CB);
+  TORCH_CHECK(lds <= 160 * 1024, "key size too large for the LDS state");
+  const int threads = CB, ncb_gen = (Dv + CB - 1) / CB;
+  TORCH_CHECK(ncb_gen <= 65535);
   SEQ_DISPATCH_ACT(q, {
     auto kern = gated_delta_scan_kernel<act_t>;
     // raise the dynamic-LDS cap once per kernel, outside any capture
@@ -545,7 +559,7 @@ void gated_delta_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
           if (p == nullptr) { p = (const void*)kern; break; }
       }
     }
-    hipLaunchKernelGGL(kern, dim3(n_seq * H), dim3(threads), lds, SEQ_STREAM(),
+    hipLaunchKernelGGL(kern, dim3(n_seq * H, ncb_gen), dim3(threads), lds, SEQ_STREAM(),
                        (float*)o.data_ptr(), (const act_t*)q.data_ptr(), q.stride(0),
                        (const act_t*)k.data_ptr(), k.stride(0),
                        (const act_t*)v.data_ptr(), v.stride(0),
@@ -554,7 +568,7 @@ void gated_delta_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                        (const float*)a_log.data_ptr(), (const float*)dt_bias.data_ptr(),
                        (float*)state.data_ptr(), (const int*)start_loc.data_ptr(),
                        (const int*)slots.data_ptr(), (const int*)positions.data_ptr(), H,
-                       G, D, Dv, (float)norm_eps);
+                       G, D, Dv, CB, (float)norm_eps);
   });
   SEQ_CHECK_LAUNCH();
 }

@@ -930,7 +930,8 @@ def test_kernel_scans_at_segment_borders(n):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 32, 16), (2, 1, 128, 40), (3, 3, 10, 6),
                                       (8, 4, 64, 64), (2, 1, 64, 8), (2, 1, 48, 24),
-                                      (1, 1, 80, 100), (2, 2, 16, 300)])
+                                      (1, 1, 80, 100), (2, 2, 16, 300), (1, 1, 200, 260),
+                                      (2, 1, 24, 70)])
 def test_kernel_delta_scan(dtype, H, G, D, Dv):
     """Register-state and LDS-state kernels, plain and segment-parallel runs,
     inputs as strided column views of one projection, against the reference."""

@@ -372,6 +372,8 @@ SINGLE = {
     "rotated_latent_no_ff": config([lat2(mlp=None)]),
     "rotated_latent_no_scaling": config([lat2(scaling=None, mlp=DENSE)]),
     "rotated_latent_one_pair": config([lat2(heads=3, dim=4, rot=2, vdim=2, rank=7, mlp=DENSE)]),
+    "rotated_latent_without_a_rotated_part": config([lat2(rot=0, mlp=DENSE)]),
+    "rotated_latent_one_head": config([lat2(heads=1, dim=8, rot=4, vdim=3, rank=5, mlp=None)]),
     "delta_no_ff": config([delta(mlp=None)]),
     "delta_every_head_its_own_key": config([delta(heads=3, kv=3, dim=8, vdim=8)]),
     "delta_one_key_head": config([delta(heads=4, kv=1, dim=16, vdim=4, conv=2)]),

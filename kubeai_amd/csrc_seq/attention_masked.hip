@@ -155,7 +155,8 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
     const T* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ token_seq,
     const int* __restrict__ positions, float scale, float softcap, int chunk,
-    int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G, int D, int Dv, int bs) {
+    int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G, int D, int Dv, int bs,
+    int kvs) {
   constexpr int N = Vec16<T>::N;
   const int lpr = kVec ? Dv / N : 1;          // lanes per value row
   const int ngrp = kVec ? WAVE / lpr : 1;     // key groups of a wave
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
       }
       sc = dot * scale;
       if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
-      vb = rowi * v_rs;
+      vb = ((blk * (G / kvs) + g / kvs) * bs + (j % bs)) * v_rs;
     }
     const float m_new = fmaxf(m, wave_max(sc));  // finite: lane 0's key is visible
     const float p = j <= pos ? expf(sc - m_new) : 0.f;
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
     int max_blocks, const int* __restrict__ start_loc,
     const int* __restrict__ positions, int tiles_per_run, float scale,
     float softcap, int chunk, int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G,
-    int D, int Dv, int bs) {
+    int D, int Dv, int bs, int kvs) {
   const int s = blockIdx.x / tiles_per_run, tile = blockIdx.x % tiles_per_run;
   const int h = blockIdx.y, g = h / (H / G);
   const int s0 = start_loc[s], s1 = start_loc[s + 1];
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
       sc[i] = vis[i] ? x : -INFINITY;
       mt = fmaxf(mt, sc[i]);
       const int jv = min(j, pos_max);
-      vrow[i] = (((int64_t)bt[jv / bs] * G + g) * bs + jv % bs) * v_rs;
+      vrow[i] = (((int64_t)bt[jv / bs] * (G / kvs) + g / kvs) * bs + jv % bs) * v_rs;
     }
     mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE));
     mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE));
@@ -444,7 +445,7 @@ __global__ __launch_bounds__(512) void masked_prefill_mfma_shared_kernel(
     int max_blocks, const int* __restrict__ start_loc,
     const int* __restrict__ positions, int tiles_per_run, float scale,
     float softcap, int chunk, int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G,
-    int D, int Dv, int bs, int HW, int QW) {
+    int D, int Dv, int bs, int HW, int QW, int kvs) {
   extern __shared__ __attribute__((aligned(16))) bf16raw lds[];
   constexpr int kKVec = kKT * kMaxDSteps * 16 / 8 / 256;   // per thread, 256 threads
   constexpr int kVVec = kKT * kMaxDvTiles * 16 / 8 / 256;
@@ -528,7 +529,7 @@ __global__ __launch_bounds__(512) void masked_prefill_mfma_shared_kernel(
       if (c < vcpr) {
         const int j = min(j0 + row, bpos_max);
         vreg[i] = *(const uint4*)(v_cache +
-            (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * v_rs + c * 8);
+            (((int64_t)bt[j / bs] * (G / kvs) + g / kvs) * bs + j % bs) * v_rs + c * 8);
       }
     }
   };
@@ -672,7 +673,7 @@ __global__ __launch_bounds__(kDW * WAVE) void masked_decode_mfma_kernel(
     int max_blocks, const int* __restrict__ token_seq,
     const int* __restrict__ positions, float scale, float softcap, int chunk,
     int window, float out_scale, const float* __restrict__ sink, int64_t v_rs, int H, int G, int D, int Dv, int bs,
-    int n_split, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int n_split, float* __restrict__ part_o, float* __restrict__ part_ml, int kvs) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int col = lane & 15, grp = lane >> 4;
@@ -710,7 +711,7 @@ __global__ __launch_bounds__(kDW * WAVE) void masked_decode_mfma_kernel(
       const int row = v % kKT, c = v / kKT;
       const int j = min(j0 + row, pos);
       const uint4 x = *(const uint4*)(v_cache +
-          (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * v_rs + c * 8);
+          (((int64_t)bt[j / bs] * (G / kvs) + g / kvs) * bs + j % bs) * v_rs + c * 8);
       const uint32_t wv[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -949,13 +950,17 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4);
   const int G = k_cache.size(1), bs = k_cache.size(2), Dv = v_cache.size(3);
-  TORCH_CHECK(k_cache.size(3) == D && v_cache.size(1) == G && v_cache.size(2) == bs);
+  // the value cache may have fewer heads than the key cache: kvs key heads
+  // (score maps over the same values) share one value head
+  const int Gv = v_cache.size(1);
+  TORCH_CHECK(k_cache.size(3) == D && Gv > 0 && G % Gv == 0 && v_cache.size(2) == bs);
+  const int kvs = G / Gv;
   // value rows may be the leading columns of wider rows (of the key rows,
   // when a layer caches one row per token that serves as both)
   const int64_t v_rs = v_cache.stride(2);
   TORCH_CHECK(v_cache.is_cuda() && (Dv == 1 || v_cache.stride(3) == 1) && v_rs >= Dv &&
               v_cache.stride(1) == (int64_t)bs * v_rs &&
-              v_cache.stride(0) == (int64_t)G * bs * v_rs,
+              v_cache.stride(0) == (int64_t)Gv * bs * v_rs,
               "value cache rows must be evenly spaced");
   const float* sink = nullptr;
   if (sink_scores.has_value()) {
@@ -991,7 +996,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
                          (const int*)positions.data_ptr(), tiles, (float)scale,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                         sink, v_rs, H, G, D, Dv, bs);
+                         sink, v_rs, H, G, D, Dv, bs, kvs);
     };
     const size_t lds_shared =
         (size_t)2 * (kKT * (D + kKPad) + Dv * (kKT + kVPad)) * sizeof(bf16raw);
@@ -1019,7 +1024,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
                          (const int*)positions.data_ptr(), btiles, (float)scale,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                         sink, v_rs, H, G, D, Dv, bs, HW, QW);
+                         sink, v_rs, H, G, D, Dv, bs, HW, QW, kvs);
       };
       // key sizes above 128 (a latent with a rotated part behind it) keep
       // twice as many query fragments in registers
@@ -1073,7 +1078,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                        (float)scale, (float)softcap, (int)chunk, (int)window,
                        (float)out_scale, sink, v_rs, H, G, D, Dv, bs, n_split,
                        n_split > 1 ? (float*)part_o.data_ptr() : nullptr,
-                       n_split > 1 ? (float*)part_ml.data_ptr() : nullptr);
+                       n_split > 1 ? (float*)part_ml.data_ptr() : nullptr, kvs);
     if (n_split > 1) {
       SEQ_CHECK_LAUNCH();
       hipLaunchKernelGGL(decode_split_join_kernel, dim3(T, H), dim3(64), 0, SEQ_STREAM(),
@@ -1106,7 +1111,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (int)block_tables.size(1), (const int*)token_seq.data_ptr(),
                          (const int*)positions.data_ptr(), (float)scale,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                         sink, v_rs, H, G, D, Dv, bs);
+                         sink, v_rs, H, G, D, Dv, bs, kvs);
     };
     if (vec) launch(masked_paged_attention_kernel<act_t, true>);
     else launch(masked_paged_attention_kernel<act_t, false>);

@@ -72,9 +72,28 @@ void latent_rope_to_cache(torch::Tensor cache, torch::Tensor x, torch::Tensor we
                           torch::Tensor slot_mapping);
 void router_scores_topk(torch::Tensor logits, c10::optional<torch::Tensor> bias,
                         torch::Tensor dense, torch::Tensor weights,
-                        torch::Tensor index);
-void silu_mul_weighted(torch::Tensor out, torch::Tensor gu, torch::Tensor w,
-                       int64_t group);
+                        torch::Tensor index, double scale);
+void glu_weighted(torch::Tensor out, torch::Tensor gu, c10::optional<torch::Tensor> w,
+                  int64_t group, double alpha, double limit, double up_shift,
+                  bool w_sigmoid);
+void embed_sinusoid(torch::Tensor out, torch::Tensor ids, torch::Tensor table,
+                    double scale, torch::Tensor positions, torch::Tensor freqs);
+void hyper_mix_rmsnorm(torch::Tensor out, torch::Tensor streams,
+                       c10::optional<torch::Tensor> y, c10::optional<torch::Tensor> gate,
+                       c10::optional<torch::Tensor> mix,
+                       c10::optional<torch::Tensor> write_w, torch::Tensor read_w,
+                       torch::Tensor weight, double eps);
+void scale_q_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                       torch::Tensor positions, double coef, int64_t every,
+                       torch::Tensor k_cache, torch::Tensor v_cache,
+                       torch::Tensor slot_mapping);
+void diff_combine(torch::Tensor out, torch::Tensor att, double lam, double gain,
+                  double eps);
+void diag_rank1_scan(torch::Tensor o, torch::Tensor r, torch::Tensor k, torch::Tensor v,
+                     torch::Tensor w_pre, torch::Tensor a_pre, torch::Tensor w_bias,
+                     torch::Tensor a_bias, torch::Tensor state, torch::Tensor start_loc,
+                     torch::Tensor slots, torch::Tensor positions, double decay_scale,
+                     double key_eps, int64_t max_len);
 void gated_delta_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                       torch::Tensor v, torch::Tensor beta_pre, torch::Tensor decay_pre,
                       torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor state,
@@ -113,7 +132,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "latent RMS norm + rotated shared key part into a paged cache, query rotation");
   m.def("router_scores_topk", &router_scores_topk,
         "softmax scores, biased top-k choice, unnormalised score weights");
-  m.def("silu_mul_weighted", &silu_mul_weighted,
-        "silu(gate) * up times a per-row, per-expert weight");
+  m.def("glu_weighted", &glu_weighted,
+        "clamped gate * sigmoid(alpha gate) * (up + shift) times a per-row, per-expert weight");
+  m.def("embed_sinusoid", &embed_sinusoid,
+        "embedding lookup + sinusoidal position vector into every residual stream");
+  m.def("hyper_mix_rmsnorm", &hyper_mix_rmsnorm,
+        "residual streams: gated write, stream mix, read, RMS norm");
+  m.def("scale_q_and_cache", &scale_q_and_cache,
+        "query temperature by position + paged cache write");
+  m.def("diff_combine", &diff_combine,
+        "difference of two attention maps + per-head RMS norm");
+  m.def("diag_rank1_scan", &diag_rank1_scan,
+        "generalized delta rule recurrence (diagonal decay + rank-one removal)");
   m.def("gated_delta_scan", &gated_delta_scan, "gated delta rule recurrence");
 }

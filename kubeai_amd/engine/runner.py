@@ -224,8 +224,9 @@ class ModelRunner:
             self.kv_dtype = dtype
         else:
             raise ValueError(f"unknown kv_cache_dtype {kv_cache_dtype!r}")
-        # per-layer cache shapes: (kv heads, key dim, value dim), or None for
-        # a layer that keeps no paged keys/values
+        # per-layer cache shapes: (kv heads, key dim, value dim[, value heads
+        # when fewer than the key heads]), or None for a layer that keeps no
+        # paged keys/values
         if hasattr(self.model, "kv_cache_specs"):
             self.kv_specs = list(self.model.kv_cache_specs())
         else:
@@ -244,7 +245,8 @@ class ModelRunner:
                     dtype=self.kv_dtype, device=self.device,
                 ),
                 torch.zeros(
-                    (num_gpu_blocks, spec[0], block_size, spec[2]),
+                    (num_gpu_blocks, spec[3] if len(spec) > 3 else spec[0], block_size,
+                     spec[2]),
                     dtype=self.kv_dtype, device=self.device,
                 ),
             )
@@ -271,7 +273,8 @@ class ModelRunner:
 
     def _profile_num_blocks(self, gpu_memory_utilization: float) -> int:
         per_block_bytes = sum(
-            spec[0] * self.block_size * (spec[1] + spec[2]) * self.kv_dtype.itemsize
+            self.block_size * (spec[0] * spec[1] + (spec[3] if len(spec) > 3 else spec[0])
+                               * spec[2]) * self.kv_dtype.itemsize
             for spec in self.kv_specs
             if spec is not None
         )

@@ -83,6 +83,8 @@ class ModelArchConfig:
             return nugopel_arch_config(cfg)
         if cfg.get("architecture") == "Vekusun":
             return vekusun_arch_config(cfg)
+        if cfg.get("architecture") == "Vigonex":
+            return vigonex_arch_config(cfg)
         hidden = cfg["hidden_size"]
         n_heads = cfg["num_attention_heads"]
         arch = (cfg.get("architectures") or ["LlamaForCausalLM"])[0]
@@ -205,6 +207,10 @@ class HybridSpec:
     # (start, stop, times): layers start..stop-1 run `times` times in a row
     # with the same weights, every pass with cache and state of its own
     loop: tuple = (0, 0, 1)
+    # residual streams (hyper-connections); 1 = one stream
+    streams: int = 1
+    # multiplier on the logits
+    logit_scale: float = 1.0
 
 
 def dulotar_arch_config(cfg: dict) -> ModelArchConfig:
@@ -306,6 +312,41 @@ def vekusun_arch_config(cfg: dict) -> ModelArchConfig:
             residual_mult=float(cfg.get("residual_mult", 1.0)),
             logit_softcap=float(cfg.get("logit_softcap") or 0.0),
             loop=(start, stop, times),
+        ),
+    )
+
+
+def vigonex_arch_config(cfg: dict) -> ModelArchConfig:
+    """Vigonex config.json -> arch config: the list of layers (mixer type, the
+    mixer's sizes and constants, the feed-forward), the number of residual
+    streams, the embedding and logit scales and the norm epsilon, all as the
+    file gives them."""
+    layers = [
+        HybridLayerSpec(type=L["type"], mixer=L["mixer"], mlp=L.get("mlp"), weights_of=i)
+        for i, L in enumerate(cfg["layers"])
+    ]
+    streams = int(cfg.get("streams", 1))
+    if streams < 1:
+        raise ValueError("streams must be at least 1")
+    return ModelArchConfig(
+        architecture="vigonex",
+        vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]),
+        num_hidden_layers=len(layers),
+        intermediate_size=0,
+        num_attention_heads=0,
+        num_key_value_heads=0,
+        head_dim=0,
+        max_position_embeddings=1 << 30,  # positions are computed, not tabulated
+        bos_token_id=-1,
+        eos_token_id=-1,  # the design defines no end token
+        hybrid=HybridSpec(
+            layers=layers,
+            norm_eps=float(cfg["norm"]["eps"]),
+            embedding_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+            canon_taps=0,
+            streams=streams,
+            logit_scale=float(cfg.get("logit_scale", 1.0)),
         ),
     )
 
@@ -821,6 +862,43 @@ def vekusun_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 
     return vekusun_arch_config(cfg)
 
 
+def vigonex_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
+                   experts: int = 8, top: int = 2, streams: int = 2,
+                   ff_scale: float = 1.0) -> ModelArchConfig:
+    """A Vigonex stack of the given size with random-init weights: the layer
+    pattern (differential attention + dense feed-forward, differential
+    attention + routed experts with a shared one, generalized delta rule +
+    routed experts, differential attention + routed experts) repeats to the
+    requested depth. Differential heads have head_dim / 2 key dims per map
+    and head_dim value dims, 4:1 grouped keys; delta heads are 64 wide. The
+    feed-forward work per token is that of a dense 3.5 x width gated layer
+    in either kind (times ff_scale, for matching another model's size)."""
+    heads = max(1, width // head_dim)
+    kv = max(1, heads // 4)
+    dim = max(8, head_dim // 2)
+    ff_dense = max(16, int(3.5 * ff_scale * width) // 16 * 16)
+    ff_exp = max(16, int(3.5 * ff_scale * width / (top + 1)) // 16 * 16)
+    dense = {"kind": "dense", "ff": ff_dense}
+    moe = {"kind": "moe", "expert": {"ff": ff_exp, "limit": 7.0},
+           "router": {"experts": experts, "top": top, "scale": 1.0},
+           "shared": {"ff": ff_exp, "limit": 7.0}}
+    att = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": head_dim, "diff": 0.3,
+           "scale": dim ** -0.5, "softcap": 30.0, "q_temp": {"coef": 0.1, "every": 1024}}
+    ddim = min(64, head_dim)
+    delta = {"heads": max(1, width // ddim), "dim": ddim, "lowrank": max(16, width // 32)}
+    pattern = [
+        {"type": "attention", "mixer": att, "mlp": dense},
+        {"type": "attention", "mixer": att, "mlp": moe},
+        {"type": "general_delta", "mixer": delta, "mlp": moe},
+        {"type": "attention", "mixer": att, "mlp": moe},
+    ]
+    return vigonex_arch_config({
+        "architecture": "Vigonex", "vocab": vocab, "width": width,
+        "norm": {"eps": 1e-6}, "streams": streams, "embedding": {"scale": 1.0},
+        "logit_scale": 1.0, "layers": [dict(pattern[i % 4]) for i in range(layers)],
+    })
+
+
 def dulotar_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
                    chunk: int = 1024, ff_mult: int = 4) -> ModelArchConfig:
     """A Dulotar stack of the given size with random-init weights: the
@@ -863,6 +941,10 @@ PRESETS.update({
     "vekusun-1k": vekusun_preset(1024, 12),
     "vekusun-2k": vekusun_preset(2048, 12),
     "vekusun-4k": vekusun_preset(4096, 6),
+    "vigonex-tiny": vigonex_preset(128, 4, vocab=512, head_dim=32, experts=4, top=2),
+    "vigonex-1k": vigonex_preset(1024, 12),
+    "vigonex-2k": vigonex_preset(2048, 12),
+    "vigonex-4k": vigonex_preset(4096, 6),
     "dulotar-tiny": dulotar_preset(128, 3, vocab=512, head_dim=32, chunk=64),
     "dulotar-1k": dulotar_preset(1024, 12),
     "dulotar-2k": dulotar_preset(2048, 12),

@@ -588,38 +588,66 @@ class RoutedSquaredReluMoE(nn.Module):
 
 
 class RoutedGatedMoE(nn.Module):
-    """Mixture of gated experts (down(silu(gate h) * (up h)), no biases).
+    """Mixture of gated experts (down(act(gate h) * (up h)), no biases).
     Routing: fp32 logits, scores = softmax over all experts; the `top`
     experts with the largest score + correction (a per-expert bias that only
-    steers the choice) are used, weighted by their scores as they are.
+    steers the choice) are used, weighted by their scores as they are (times
+    weight_scale).
+
+    The activation is g * sigmoid(act_alpha * g) * (u + up_shift), with
+    g = min(gate, act_limit) and u = clamp(up, +-act_limit) when act_limit > 0
+    (defaults: silu(gate) * up). shared_ff > 0 adds one expert of that size
+    that every token uses (its own clamp shared_limit), weighted by the
+    sigmoid of one more router row when shared_gate is set.
 
     Expert e's gate and up matrices are rows [e*2ff, e*2ff + ff) and
-    [e*2ff + ff, (e+1)*2ff) of one stacked matrix, all down-projections one
-    [width, E*ff]. Small steps (decode) run two GEMMs over every expert with
-    the routing weight (0 for experts a token did not choose) folded into the
-    activation, so the weighted sum happens inside the second GEMM's fp32
-    accumulation and the step has no data-dependent shapes. Large steps
-    gather each expert's tokens and run its slice."""
+    [e*2ff + ff, (e+1)*2ff) of one stacked matrix (the shared expert's follow
+    them), all down-projections one [width, E*ff + shared_ff]. Small steps
+    (decode) run two GEMMs over every expert with the routing weight (0 for
+    experts a token did not choose) folded into the activation, so the
+    weighted sum happens inside the second GEMM's fp32 accumulation and the
+    step has no data-dependent shapes. Large steps gather each expert's
+    tokens and run its slice."""
 
     DENSE_MAX_TOKENS = 256
 
-    def __init__(self, width, experts, top, ff, correction=True):
+    def __init__(self, width, experts, top, ff, correction=True, act_alpha=1.0,
+                 act_limit=0.0, up_shift=0.0, weight_scale=1.0, shared_ff=0,
+                 shared_limit=0.0, shared_gate=False):
         super().__init__()
         self.experts, self.top, self.ff = experts, top, ff
-        self.router = nn.Parameter(torch.empty(experts, width, dtype=torch.float32),
-                                   requires_grad=False)
+        self.act = dict(alpha=float(act_alpha), limit=float(act_limit or 0.0),
+                        up_shift=float(up_shift))
+        self.weight_scale = float(weight_scale)
+        self.shared_ff = int(shared_ff or 0)
+        self.shared_act = dict(self.act, limit=float(shared_limit or 0.0))
+        self.shared_gate = bool(shared_gate) and self.shared_ff > 0
+        # the shared expert's gate is one more row behind the experts'
+        self.router = nn.Parameter(
+            torch.empty(experts + int(self.shared_gate), width, dtype=torch.float32),
+            requires_grad=False)
         nn.init.normal_(self.router, std=width ** -0.5)
         self.correction = _f32(experts) if correction else None
-        self.gate_up = Proj(width, experts * 2 * ff)
-        self.down = Proj(experts * ff, width)
+        self.gate_up = Proj(width, experts * 2 * ff + 2 * self.shared_ff)
+        self.down = Proj(experts * ff + self.shared_ff, width)
 
     def forward(self, h):
         T = h.shape[0]
-        E, ff = self.experts, self.ff
+        E, ff, sff = self.experts, self.ff, self.shared_ff
         logits = F.linear(h.float(), self.router)
-        dense, w, idx = sops.router_scores_topk(logits, self.top, self.correction)
+        sg = logits[:, E:] if self.shared_gate else None
+        dense, w, idx = sops.router_scores_topk(
+            logits[:, :E] if self.shared_gate else logits, self.top, self.correction,
+            self.weight_scale)
         if T <= self.DENSE_MAX_TOKENS:
-            return self.down(sops.silu_mul_weighted(self.gate_up(h), dense, ff))
+            gu = self.gate_up(h)
+            a = torch.empty((T, E * ff + sff), dtype=h.dtype, device=h.device)
+            sops.glu_weighted(gu[:, : E * 2 * ff], dense, ff, out=a[:, : E * ff],
+                              **self.act)
+            if sff:
+                sops.glu_weighted(gu[:, E * 2 * ff :], sg, sff, w_sigmoid=True,
+                                  out=a[:, E * ff :], **self.shared_act)
+            return self.down(a)
         out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
         flat = idx.flatten().long()
         order = torch.argsort(flat, stable=True)
@@ -634,8 +662,172 @@ class RoutedGatedMoE(nn.Module):
             rows = tok[s : s + n]
             gu = F.linear(h.index_select(0, rows),
                           self.gate_up.weight[e * 2 * ff : (e + 1) * 2 * ff])
-            a = sops.silu_mul_weighted(gu, wrow[s : s + n], ff)
+            a = sops.glu_weighted(gu, wrow[s : s + n], ff, **self.act)
             y = F.linear(a, self.down.weight[:, e * ff : (e + 1) * ff])
             out.index_add_(0, rows, y.float())
             s += n
+        if sff:
+            gu = F.linear(h, self.gate_up.weight[E * 2 * ff :])
+            a = sops.glu_weighted(gu, sg, sff, w_sigmoid=True, **self.shared_act)
+            out.add_(F.linear(a, self.down.weight[:, E * ff :]))
         return out
+
+
+class SiluGatedMLP(nn.Module):
+    """Dense gated feed-forward: down(silu(gate h) * (up h)); the gate and up
+    matrices are one stacked [2 ff, width] product."""
+
+    def __init__(self, width: int, ff: int):
+        super().__init__()
+        self.ff = ff
+        self.gate_up = Proj(width, 2 * ff)
+        self.down = Proj(ff, width)
+
+    def forward(self, h):
+        return self.down(sops.glu_weighted(self.gate_up(h), None, self.ff))
+
+
+class BiasProj(nn.Module):
+    """Linear layer [out, in] with a bias, both in the serving dtype (the
+    bias is added in the product's epilogue)."""
+
+    def __init__(self, n_in: int, n_out: int):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(n_out, n_in), requires_grad=False)
+        nn.init.normal_(self.weight, std=n_in ** -0.5)
+        self.bias = nn.Parameter(torch.zeros(n_out), requires_grad=False)
+
+    def forward(self, x):
+        return F.linear(x, self.weight, self.bias)
+
+
+class DifferentialAttention(nn.Module):
+    """Causal softmax attention in which every query head computes two score
+    maps (two query and two key vectors per head) over the same values and
+    outputs their difference, map 1 - lam * map 2, RMS-normed per head
+    (no weight) and scaled by `gain`. Grouped key/value heads, separate key
+    and value sizes, a tanh cap on the scores, biases on every projection.
+    Positions enter only through a query temperature
+    1 + coef * ln(floor((p + 1) / every) + 1) (coef 0: none).
+
+    lam is one number for the layer: exp(lq1 . lk1) - exp(lq2 . lk2) + lam0.
+
+    The two maps are ordinary attention heads to the kernels: the cache keeps
+    2 G key heads (head 2 g + m is map m of group g) and G value heads; the
+    query rows are ordered (group, map, head in group), so that query head j
+    reads key head j // R and value head j // 2R (R = heads per group)."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, softcap=0.0,
+                 lam0=0.0, gain=1.0, temp_coef=0.0, temp_every=1, eps=1e-6):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.softcap = float(scale), float(softcap or 0.0)
+        self.lam0, self.gain, self.eps = float(lam0), float(gain), eps
+        self.temp_coef, self.temp_every = float(temp_coef or 0.0), max(1, int(temp_every))
+        self.sizes = (2 * heads * dim, 2 * kv_heads * dim, kv_heads * vdim)
+        self.in_proj = BiasProj(width, sum(self.sizes))  # q | k | v
+        self.o_proj = BiasProj(heads * vdim, width)
+        self.lam_q = _f32(2, dim)
+        self.lam_k = _f32(2, dim)
+        self._lam = None
+
+    def state_spec(self):
+        return {}
+
+    def kv_spec(self):
+        # (key heads, key size, value size, value heads)
+        return (2 * self.kv_heads, self.dim, self.vdim, self.kv_heads)
+
+    def query_row_order(self):
+        """Index of the checkpoint's query rows (head, map, dim) in the
+        engine's order (group, map, head in group, dim)."""
+        H, G, D = self.heads, self.kv_heads, self.dim
+        idx = torch.arange(2 * H * D).view(G, H // G, 2, D)
+        return idx.permute(0, 2, 1, 3).reshape(-1)
+
+    @property
+    def lam(self) -> float:
+        if self._lam is None:
+            dots = (self.lam_q.double() * self.lam_k.double()).sum(-1).float()
+            e = torch.exp(dots)
+            self._lam = float(e[0] - e[1]) + self.lam0
+        return self._lam
+
+    def forward(self, h, fb, state, kv_cache):
+        T = h.shape[0]
+        H, G, D, Dv = self.heads, self.kv_heads, self.dim, self.vdim
+        nq, nk, _ = self.sizes
+        qkv = self.in_proj(h)
+        q = qkv[:, :nq].unflatten(-1, (2 * H, D))
+        k = qkv[:, nq : nq + nk].unflatten(-1, (2 * G, D))
+        v = qkv[:, nq + nk :].unflatten(-1, (G, Dv))
+        k_cache, v_cache = kv_cache
+        sops.scale_q_and_cache(q, k, v, fb.positions, self.temp_coef, self.temp_every,
+                               k_cache, v_cache, fb.slot_mapping)
+        att = torch.empty((T, 2 * H, Dv), dtype=h.dtype, device=h.device)
+        sops.masked_paged_attention(q, k_cache, v_cache, fb.seq, self.scale, att,
+                                    softcap=self.softcap)
+        out = torch.empty((T, H, Dv), dtype=h.dtype, device=h.device)
+        sops.diff_combine(att.view(T, G, 2, H // G, Dv), self.lam, self.gain, self.eps,
+                          out)
+        return self.o_proj(out.view(T, H * Dv))
+
+
+class GeneralDeltaMixer(nn.Module):
+    """Generalized delta rule: a matrix state per head with a per-channel,
+    data-dependent decay (through a low-rank tanh bottleneck) and a
+    per-channel removal rate along the unit key:
+    S <- diag(w) S - (a * n)(n^T S) + k v^T, o = S^T r (ops.seq.diag_rank1_scan).
+    r, k, v have heads x dim channels; the read-out is RMS-normed per head,
+    times a weight over all heads, times sigmoid of a gate projection."""
+
+    def __init__(self, width, heads, dim, lowrank, eps, decay_scale=0.6065306597126334,
+                 key_eps=1e-6):
+        super().__init__()
+        self.heads, self.dim, self.lowrank, self.eps = heads, dim, int(lowrank), eps
+        self.decay_scale, self.key_eps = float(decay_scale), float(key_eps)
+        n = heads * dim
+        self.in_proj = Proj(width, 5 * n + self.lowrank)  # r | k | v | g | a | w1
+        self.w2 = Proj(self.lowrank, n)
+        self.w0 = _f32(n)
+        self.a_bias = _f32(n)
+        self.norm = _f32(n)
+        nn.init.ones_(self.norm)
+        self.o_proj = Proj(n, width)
+
+    def set_lowrank(self, lowrank: int):
+        """Resize the decay bottleneck (a checkpoint gives its size by the
+        shape of its tensors)."""
+        if int(lowrank) == self.lowrank:
+            return
+        n, w = self.heads * self.dim, self.in_proj.weight
+        self.lowrank = int(lowrank)
+        self.in_proj.weight = nn.Parameter(
+            torch.zeros((5 * n + self.lowrank, w.shape[1]), dtype=w.dtype, device=w.device),
+            requires_grad=False)
+        self.w2.weight = nn.Parameter(
+            torch.zeros((n, self.lowrank), dtype=w.dtype, device=w.device),
+            requires_grad=False)
+
+    def state_spec(self):
+        return {"s": (self.heads, self.dim, self.dim)}
+
+    def kv_spec(self):
+        return None
+
+    def forward(self, h, fb, state, kv_cache):
+        T = h.shape[0]
+        H, D = self.heads, self.dim
+        n = H * D
+        proj = self.in_proj(h)
+        w_pre = self.w2(torch.tanh(proj[:, 5 * n :]))
+        part = lambda i: proj[:, i * n : (i + 1) * n].unflatten(-1, (H, D))
+        o = sops.diag_rank1_scan(part(0), part(1), part(2), w_pre.view(T, H, D), part(4),
+                                 self.w0, self.a_bias, state["s"], fb.seq,
+                                 self.decay_scale, self.key_eps)
+        y = torch.empty((T, n), dtype=h.dtype, device=h.device)
+        sops.gated_rmsnorm(o.view(T, n), self.norm, proj[:, 3 * n : 4 * n], H, "sigmoid",
+                           self.eps, y)
+        return self.o_proj(y)

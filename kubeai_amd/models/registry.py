@@ -27,12 +27,19 @@ def _vekusun():
     return VekusunForCausalLM
 
 
+def _vigonex():
+    from .vigonex import VigonexForCausalLM
+
+    return VigonexForCausalLM
+
+
 MODEL_REGISTRY = {
     "llama": _llama,
     "mixtral": _llama,
     "dulotar": _dulotar,
     "nugopel": _nugopel,
     "vekusun": _vekusun,
+    "vigonex": _vigonex,
 }
 
 
@@ -53,6 +60,7 @@ MODEL_EXTENSIONS = {
     "dulotar": ("_C_seq",),
     "nugopel": ("_C_seq",),
     "vekusun": ("_C_seq",),
+    "vigonex": ("_C_seq",),
 }
 
 

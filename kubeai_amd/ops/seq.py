@@ -645,11 +645,11 @@ def relu_squared_weighted(u, w, group: int):
     return r.to(u.dtype)
 
 
-def router_scores_topk(logits, top: int, bias=None):
+def router_scores_topk(logits, top: int, bias=None, scale: float = 1.0):
     """Routing by scores: s = softmax(logits) over all experts (fp32); the
     `top` experts with the largest s + bias are chosen (equal values: lower
     index first; bias fp32 [E] or None), and their weights are their scores
-    s themselves, not renormalised. Returns (dense [T, E] with the weights at
+    s themselves times `scale`, not renormalised. Returns (dense [T, E] with the weights at
     the chosen experts' columns, weights [T, top], index int32 [T, top])."""
     T, E = logits.shape
     if logits.is_cuda:
@@ -657,12 +657,12 @@ def router_scores_topk(logits, top: int, bias=None):
         dense = torch.empty((T, E), dtype=torch.float32, device=logits.device)
         w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
         idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
-        _C.router_scores_topk(logits.contiguous(), bias, dense, w, idx)
+        _C.router_scores_topk(logits.contiguous(), bias, dense, w, idx, scale)
         return dense, w, idx
     s = torch.softmax(logits.float(), dim=-1)
     choice = s if bias is None else s + bias
     idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
-    w = torch.gather(s, 1, idx)
+    w = torch.gather(s, 1, idx) * scale
     dense = torch.zeros((T, E), dtype=torch.float32)
     dense.scatter_(1, idx, w)
     return dense, w, idx.to(torch.int32)
@@ -673,16 +673,39 @@ def silu_mul_weighted(gu, w, group: int):
     [T, n * 2 * group] holds, per expert e, `group` gate columns followed by
     `group` up columns; out[t, e * group + c] = silu(gate) * up * w[t, e].
     w fp32 [T, n] (a strided column view is fine)."""
+    return glu_weighted(gu, w, group)
+
+
+def glu_weighted(gu, w, group: int, *, alpha: float = 1.0, limit: float = 0.0,
+                 up_shift: float = 0.0, w_sigmoid: bool = False, out=None):
+    """Gated activation over blocks of `group` gate columns followed by
+    `group` up columns (gu [T, n * 2 * group], rows may be strided):
+
+        g = gate, u = up;  with limit > 0: g = min(g, limit), u = clamp(u, -limit, limit)
+        out[t, e * group + c] = g * sigmoid(alpha * g) * (u + up_shift) * w[t, e]
+
+    alpha = 1 is silu. w fp32 [T, n] (strided columns view fine) or None (no
+    weight); with w_sigmoid the weight is sigmoid(w). out [T, n * group] may
+    be a strided column view of a wider buffer. fp32 inside."""
     T, C2 = gu.shape
     n = C2 // (2 * group)
+    if out is None:
+        out = torch.empty((T, n * group), dtype=gu.dtype, device=gu.device)
     if gu.is_cuda:
         _require_ext()
-        out = torch.empty((T, n * group), dtype=gu.dtype, device=gu.device)
-        _C.silu_mul_weighted(out, gu, w, group)
+        _C.glu_weighted(out, gu, w, group, alpha, limit, up_shift, w_sigmoid)
         return out
-    g = gu.float().view(T, n, 2, group)
-    a = g[:, :, 0] * torch.sigmoid(g[:, :, 0]) * g[:, :, 1] * w.unsqueeze(-1)
-    return a.reshape(T, n * group).to(gu.dtype)
+    g = gu.float().reshape(T, n, 2, group)
+    gate, up = g[:, :, 0], g[:, :, 1]
+    if limit > 0:
+        gate = gate.clamp(max=limit)
+        up = up.clamp(-limit, limit)
+    a = gate * torch.sigmoid(alpha * gate) * (up + up_shift)
+    if w is not None:
+        wf = torch.sigmoid(w.float()) if w_sigmoid else w.float()
+        a = a * wf.unsqueeze(-1)
+    out.copy_(a.reshape(T, n * group).to(out.dtype))
+    return out
 
 
 # ---------------------------------------------------------------------------
@@ -702,7 +725,10 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
     sink[h] as it stands (not scaled, not capped) and that carries no value:
     the denominator grows by exp(sink[h]).
     q [T, H, D] (strided ok), caches [blocks, G, block, D | Dv]; v_cache may
-    be the leading Dv columns of the key rows (a view of k_cache);
+    be the leading Dv columns of the key rows (a view of k_cache), or have
+    fewer heads than k_cache (Gv dividing G: query head h reads key head
+    h // (H / G) and value head h // (H / Gv), so several score maps share
+    one value head);
     out [T, H, Dv] may be a strided view; out = attention * out_scale.
     sink=True stands for a score of 0 on every head."""
     if sink is True:
@@ -718,7 +744,7 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
         return out
     T, H, D = q.shape
     G, bs = k_cache.shape[1], k_cache.shape[2]
-    rep = H // G
+    rep, rep_v = H // G, H // v_cache.shape[1]
     bt = meta.block_tables
     sl = meta.start_loc.tolist()
     for si in range(meta.n_seq):
@@ -737,7 +763,7 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
         ks = k_cache[blk, :, j % bs].float()  # [L', G, D]
         vs = v_cache[blk, :, j % bs].float()
         ks = ks.repeat_interleave(rep, dim=1)
-        vs = vs.repeat_interleave(rep, dim=1)
+        vs = vs.repeat_interleave(rep_v, dim=1)
         s = torch.einsum("thd,lhd->htl", q[s0 : s0 + n].float(), ks) * scale
         if softcap > 0:
             s = softcap * torch.tanh(s / softcap)
@@ -756,3 +782,144 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
         o = torch.einsum("htl,lhd->thd", p, vs) * out_scale
         out[s0 : s0 + n] = o.to(out.dtype)
     return out
+
+
+# ---------------------------------------------------------------------------
+# sinusoidal positions, residual streams, differential attention, the
+# generalized delta rule
+# ---------------------------------------------------------------------------
+
+def embed_sinusoid(ids, table, scale: float, positions, freqs, copies: int = 1):
+    """fp32 [T, copies, C], every copy table[ids] * scale plus a position
+    vector whose column c is sin (c even) or cos (c odd) of
+    position * freqs[c // 2] (fp32 angle). table [V, C] in the serving dtype,
+    freqs fp32 [ceil(C / 2)]."""
+    T, C = ids.shape[0], table.shape[1]
+    if table.is_cuda:
+        _require_ext()
+        out = torch.empty((T, copies, C), dtype=torch.float32, device=table.device)
+        _C.embed_sinusoid(out, ids, table, scale, positions, freqs)
+        return out
+    ang = positions.float().unsqueeze(-1) * freqs  # [T, ceil(C/2)]
+    pe = torch.stack([torch.sin(ang), torch.cos(ang)], dim=-1).reshape(T, -1)[:, :C]
+    x = table[ids.long()].float() * scale + pe
+    return x.unsqueeze(1).repeat(1, copies, 1)
+
+
+def hyper_mix_rmsnorm(streams, y, gate, mix, out_w, in_w, weight, eps: float,
+                      out_dtype):
+    """Residual streams (hyper-connections) around a sublayer, fused with the
+    next sublayer's input norm. streams fp32 [T, S, C], updated in place:
+
+        z = y * sigmoid(gate)                  (gate None: z = y)
+        streams[:, t] <- sum_s mix[s, t] streams[:, s] + out_w[t] * z
+        u = sum_s in_w[s] streams[:, s]
+        returns u / sqrt(mean(u^2) + eps) * weight      (out_dtype)
+
+    y [T, C] is the previous sublayer's output (serving dtype or fp32; None:
+    the streams stay as they are), gate [T, C] its gate's pre-activation (rows
+    may be strided), mix fp32 [S, S] indexed [from, to], out_w and in_w fp32
+    [S], weight fp32 [C]. All sums are fp32."""
+    if streams.is_cuda:
+        _require_ext()
+        out = torch.empty((streams.shape[0], streams.shape[2]), dtype=out_dtype,
+                          device=streams.device)
+        _C.hyper_mix_rmsnorm(out, streams, y, gate, mix, out_w, in_w, weight, eps)
+        return out
+    if y is not None:
+        z = y.float()
+        if gate is not None:
+            z = z * torch.sigmoid(gate.float())
+        new = torch.einsum("st,nsc->ntc", mix, streams) + out_w.view(1, -1, 1) * z.unsqueeze(1)
+        streams.copy_(new)
+    u = torch.einsum("s,nsc->nc", in_w, streams)
+    return (u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * weight).to(out_dtype)
+
+
+def scale_q_and_cache(q, k, v, positions, coef: float, every: int, k_cache,
+                      v_cache, slot_mapping):
+    """Position-dependent query temperature fused with the paged cache write:
+    q[t] *= 1 + coef * ln(floor((p + 1) / every) + 1) at position p (fp32; in
+    place; coef 0 leaves q alone); k and v rows go to their caches at
+    slot_mapping (slot < 0: no write). q [T, H, D], k [T, G, D], v [T, Gv, Dv]
+    may be strided views; the caches are [blocks, G | Gv, block, D | Dv]."""
+    if q.is_cuda:
+        _require_ext()
+        _C.scale_q_and_cache(q, k, v, positions, coef, every, k_cache, v_cache,
+                             slot_mapping)
+        return q
+    if coef != 0.0:
+        p = positions.long()
+        temp = 1.0 + coef * torch.log(
+            torch.div(p + 1, int(every), rounding_mode="floor").float() + 1.0)
+        q.copy_((q.float() * temp.view(-1, 1, 1)).to(q.dtype))
+    bs = k_cache.shape[2]
+    ok = slot_mapping >= 0
+    blk = (slot_mapping[ok] // bs).long()
+    off = (slot_mapping[ok] % bs).long()
+    k_cache[blk, :, off] = k[ok].to(k_cache.dtype)
+    v_cache[blk, :, off] = v[ok].to(v_cache.dtype)
+    return q
+
+
+def diff_combine(att, lam: float, gain: float, eps: float, out):
+    """Differential attention's join: att [T, G, 2, R, Dv] holds, per group
+    of R query heads, the outputs of the two softmax maps; for head (g, r)
+
+        o = att[:, g, 0, r] - lam * att[:, g, 1, r]
+        out[:, g * R + r] = o / sqrt(mean(o^2) + eps) * gain
+
+    in fp32. out [T, G * R, Dv] may be a strided view."""
+    T, G, _, R, Dv = att.shape
+    if att.is_cuda:
+        _require_ext()
+        _C.diff_combine(out, att, lam, gain, eps)
+        return out
+    a = att.float()
+    o = a[:, :, 0] - lam * a[:, :, 1]
+    o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * gain
+    out.copy_(o.reshape(T, G * R, Dv).to(out.dtype))
+    return out
+
+
+def diag_rank1_scan(r, k, v, w_pre, a_pre, w_bias, a_bias, state, meta: SeqMeta,
+                    decay_scale: float, key_eps: float = 1e-6):
+    """Generalized delta rule: per head a matrix state S [D, Dv] (fp32) whose
+    transition is a diagonal decay plus a rank-one removal along the unit key,
+    both applied to the old state, followed by the write:
+
+        w = exp(-decay_scale * sigmoid(w_pre + w_bias)),  a = sigmoid(a_pre + a_bias)
+        n = k / sqrt(|k|^2 + key_eps)
+        S <- diag(w) S - (a * n) (n^T S) + k v^T;   o = S^T r
+
+    r, k, w_pre, a_pre [T, H, D], v [T, H, Dv] (strided column views of one
+    projection are fine), w_bias, a_bias fp32 [H * D], state fp32
+    [slots, H, D, Dv]. Everything but the loads is fp32. Returns o fp32
+    [T, H, Dv]."""
+    T, H, D = k.shape
+    Dv = v.shape[2]
+    if k.is_cuda:
+        _require_ext()
+        o = torch.empty((T, H, Dv), dtype=torch.float32, device=k.device)
+        _C.diag_rank1_scan(o, r, k, v, w_pre, a_pre, w_bias, a_bias, state,
+                           meta.start_loc, meta.slots, meta.positions, decay_scale,
+                           key_eps, meta.max_len)
+        return o
+    o = torch.empty((T, H, Dv), dtype=torch.float32)
+    for s0, n, slot, p0 in meta.runs():
+        rs, ks, vs = (x[s0 : s0 + n].float() for x in (r, k, v))
+        w = torch.exp(-decay_scale * torch.sigmoid(
+            w_pre[s0 : s0 + n].float() + w_bias.view(H, D)))
+        a = torch.sigmoid(a_pre[s0 : s0 + n].float() + a_bias.view(H, D))
+        un = ks * torch.rsqrt((ks * ks).sum(-1, keepdim=True) + key_eps)
+        S = (state[slot].clone() if (slot >= 0 and p0 > 0)
+             else torch.zeros(H, D, Dv))
+        for t in range(n):
+            proj = torch.einsum("hk,hkv->hv", un[t], S)
+            S = (w[t].unsqueeze(-1) * S
+                 - (a[t] * un[t]).unsqueeze(-1) * proj.unsqueeze(-2)
+                 + ks[t].unsqueeze(-1) * vs[t].unsqueeze(-2))
+            o[s0 + t] = torch.einsum("hkv,hk->hv", S, rs[t])
+        if slot >= 0:
+            state[slot] = S
+    return o

@@ -179,3 +179,80 @@ def forward(cfg, W, tokens, layers_out=None):
             layers_out.append(X.sum(0))
     h = unit_rms(X.sum(0), eps) * W["final.norm"]
     return (h @ W["head"].T) * float(cfg.get("logit_scale", 1.0))
+
+
+def random_weights(cfg, seed):
+    """{name: bfloat16 torch tensor} for a config; the decay bottleneck of a
+    delta layer has mixer["lowrank"] rows (default 5)."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    W = {}
+
+    def mat(name, n_out, n_in, gain=1.0):
+        W[name] = (torch.randn(n_out, n_in, generator=g) * gain * n_in ** -0.5).bfloat16()
+
+    def vec(name, n, center, spread=0.2):
+        W[name] = (center + spread * torch.randn(n, generator=g)).bfloat16()
+
+    width, vocab, S = cfg["width"], cfg["vocab"], int(cfg.get("streams", 1))
+    W["embed"] = torch.randn(vocab, width, generator=g).bfloat16()
+    mat("head", vocab, width, 2.0)
+    vec("final.norm", width, 1.0)
+    for i, L in enumerate(cfg["layers"]):
+        p, mx, q = f"l{i}.", L["mixer"], f"l{i}.mix."
+        W[p + "shift"] = torch.rand(width, generator=g).bfloat16()
+        for n in (1, 2):
+            if n == 2 and L.get("mlp") is None:
+                continue
+            vec(f"{p}norm{n}", width, 1.0)
+            vec(f"{p}hc{n}.in", S, 1.0 / S, 0.3)
+            vec(f"{p}hc{n}.out", S, 1.0, 0.4)
+            W[f"{p}hc{n}.mix"] = (torch.eye(S) + 0.3 * torch.randn(S, S, generator=g)).bfloat16()
+            mat(f"{p}rg{n}", width, width, 2.0)
+            vec(f"{p}rg{n}.b", width, 0.5, 1.0)
+        if L["type"] == "attention":
+            H, G, D, Dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+            for name, n_out in (("q", 2 * H * D), ("k", 2 * G * D), ("v", G * Dv)):
+                mat(q + name, n_out, width, 2.0)
+                vec(q + name + ".b", n_out, 0.0, 0.3)
+            for name in ("lq1", "lk1", "lq2", "lk2"):
+                vec(q + name, D, 0.0, 0.5 * D ** -0.5)
+            mat(q + "o", width, H * Dv)
+            vec(q + "o.b", width, 0.0, 0.3)
+        else:
+            H, D = mx["heads"], mx["dim"]
+            R = int(mx.get("lowrank", 5))
+            for name in "rkvga":
+                mat(q + name, H * D, width, 2.0)
+            vec(q + "a.b", H * D, 0.0, 1.0)
+            mat(q + "w1", R, width, 2.0)
+            mat(q + "w2", H * D, R, 2.0)
+            vec(q + "w0", H * D, -0.5, 1.5)
+            vec(q + "norm", H * D, 1.0)
+            mat(q + "o", width, H * D)
+        mlp = L.get("mlp")
+        if mlp is None:
+            continue
+        q = p + "mlp."
+        if mlp["kind"] == "dense":
+            mat(q + "gate", mlp["ff"], width, 2.0)
+            mat(q + "up", mlp["ff"], width, 2.0)
+            mat(q + "down", width, mlp["ff"])
+        else:
+            names = [f"{q}e{e}." for e in range(mlp["router"]["experts"])]
+            sizes = [mlp["expert"]["ff"]] * len(names)
+            if mlp.get("shared"):
+                names.append(q + "shared.")
+                sizes.append(mlp["shared"]["ff"])
+                mat(q + "shared.sg", 1, width, 3.0)
+            for n, ff in zip(names, sizes):
+                mat(n + "gate", ff, width, 3.0)
+                mat(n + "up", ff, width, 3.0)
+                mat(n + "down", width, ff)
+            mat(q + "router", mlp["router"]["experts"], width, 4.0)
+    return W
+
+
+def as_float64(W):
+    return {k: v.double().numpy() for k, v in W.items()}

@@ -94,7 +94,7 @@ def get_args():
                    "throughput of a layer-list design beside the closest "
                    "equal-size Llama-family stack (benchmarks/hybrid_compare.py)")
     p.add_argument("--compare-design", default="dulotar",
-                   choices=["dulotar", "nugopel", "vekusun"],
+                   choices=["dulotar", "nugopel", "vekusun", "vigonex"],
                    help="which design --compare-hybrid measures")
     p.add_argument("--compare-sizes", default="1k,2k,4k")
     return p.parse_args()

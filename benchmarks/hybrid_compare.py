@@ -1,11 +1,13 @@
 """Prefill and decode throughput of a layer-list design (Dulotar, Nugopel,
-Vekusun) beside the closest existing stack of equal width, depth and (about)
-parameter count, random weights, one GPU: a dense Llama for Dulotar, a
-Mixtral-style routed Llama (same number of experts and choices) for Nugopel,
-and Nugopel itself (latent attention, routed experts) for Vekusun, whose
-feed-forward sizes are scaled so that the parameter counts agree.
+Vekusun, Vigonex) beside the closest existing stack of equal width, depth and
+(about) parameter count, random weights, one GPU: a dense Llama for Dulotar,
+a Mixtral-style routed Llama (same number of experts and choices) for
+Nugopel, Nugopel itself (latent attention, routed experts) for Vekusun, and
+Vekusun (full causal attention, a delta rule, dense and routed gated
+feed-forwards, sequence state) for Vigonex; the feed-forward sizes of the
+last two are scaled so that the parameter counts agree.
 
-    python bench.py --compare-hybrid [--compare-design dulotar|nugopel|vekusun]
+    python bench.py --compare-hybrid [--compare-design dulotar|nugopel|vekusun|vigonex]
                     [--compare-sizes 1k,2k,4k]
 
 Prefill: one sequence's whole prompt as a single fixed step (both families
@@ -66,15 +68,19 @@ def _meta_params(arch: ModelArchConfig) -> int:
     return _params(model_class(arch.architecture)(arch, device="meta"))
 
 
+def _sized_like(preset, width: int, layers: int, target_params: int) -> ModelArchConfig:
+    """preset(width, layers, ff_scale=...) with its feed-forward sizes scaled
+    to the target parameter count (the count is linear in the scale)."""
+    p1 = _meta_params(preset(width, layers, ff_scale=1.0))
+    p2 = _meta_params(preset(width, layers, ff_scale=2.0))
+    scale = 1.0 + (target_params - p1) / max(p2 - p1, 1)
+    return preset(width, layers, ff_scale=max(scale, 0.1))
+
+
 def _vekusun_sized_like(width: int, layers: int, target_params: int) -> ModelArchConfig:
-    """The Vekusun preset of this width and depth with its feed-forward sizes
-    scaled to the target parameter count (the count is linear in the scale)."""
     from kubeai_amd.models.config import vekusun_preset
 
-    p1 = _meta_params(vekusun_preset(width, layers, ff_scale=1.0))
-    p2 = _meta_params(vekusun_preset(width, layers, ff_scale=2.0))
-    scale = 1.0 + (target_params - p1) / max(p2 - p1, 1)
-    return vekusun_preset(width, layers, ff_scale=max(scale, 0.1))
+    return _sized_like(vekusun_preset, width, layers, target_params)
 
 
 def _engine(name: str, device: str, blocks: int, seqs: int, max_len: int):
@@ -140,7 +146,7 @@ def main(args) -> None:
     prefill_lens = [2048, 8192] if device == "cuda" else [64]
     batches = [(64, 1536), (8, 3584)] if device == "cuda" else [(2, 32)]
     design = getattr(args, "compare_design", None) or "dulotar"
-    if design not in ("dulotar", "nugopel", "vekusun"):
+    if design not in ("dulotar", "nugopel", "vekusun", "vigonex"):
         raise SystemExit(f"unknown design {design!r}")
     for key in sizes:
         width, layers = SIZES[key]
@@ -149,6 +155,12 @@ def main(args) -> None:
             name = f"vekusun-like-nugopel-{key}"
             PRESETS[name] = _vekusun_sized_like(
                 width, layers, _meta_params(PRESETS[f"nugopel-{key}"]))
+        if design == "vigonex" and device == "cuda":
+            from kubeai_amd.models.config import vigonex_preset
+
+            name = f"vigonex-like-vekusun-{key}"
+            PRESETS[name] = _sized_like(vigonex_preset, width, layers,
+                                        _meta_params(PRESETS[f"vekusun-{key}"]))
         arch = PRESETS[name]
         max_len = 8192 + 256
         blocks = (max(b * (c + 128) for b, c in batches) + max_len) // 16 + 64
@@ -161,6 +173,9 @@ def main(args) -> None:
         if design == "vekusun":
             ref_fam = "nugopel"
             ref_name = f"nugopel-{key}" if device == "cuda" else "nugopel-tiny"
+        elif design == "vigonex":
+            ref_fam = "vekusun"
+            ref_name = f"vekusun-{key}" if device == "cuda" else "vekusun-tiny"
         elif moe:
             ref_fam = "mixtral"
             PRESETS[ref_name] = _llama_like(

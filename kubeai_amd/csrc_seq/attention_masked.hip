@@ -1043,9 +1043,11 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
     SEQ_CHECK_LAUNCH();
     return;
   }
-  // worth it when many heads share a row (measured: 16 heads on one latent
-  // 60 -> 28 us per call, groups of 4 no faster than the generic kernel)
-  if (q.scalar_type() == torch::kBFloat16 && max_len == 1 && H / G >= 8 && D % 16 == 0 &&
+  // worth it when several heads share a key row (measured at 64 sequences of
+  // 1536 tokens: 16 heads on one latent 60 -> 28 us per call; groups of 4 with
+  // 128-wide keys 89 -> 65 us, with two 64-wide score maps per value head
+  // 132 -> 93 us)
+  if (q.scalar_type() == torch::kBFloat16 && max_len == 1 && H / G >= 4 && D % 16 == 0 &&
       Dv % 16 == 0 && D <= 256 && Dv <= 128 && al8(q) && v_rs % 8 == 0 &&
       ((size_t)k_cache.data_ptr()) % 16 == 0 && ((size_t)v_cache.data_ptr()) % 16 == 0) {
     // decode tokens: the heads of a key/value group are the rows of a tile

@@ -11,18 +11,22 @@ constexpr int kBlock = 256;
 constexpr int kMaxStreams = 8;
 
 // grid (T). out[t, s, c] = table[id, c] * scale + (c odd ? cos : sin)(pos * freqs[c / 2])
-// for every stream s. The angle is an fp32 product, sinf / cosf are the
-// precise library functions.
+// for every stream s. The angle is formed and reduced to [0, 2 pi) in double
+// (an fp32 product loses the phase at positions in the thousands); sinf /
+// cosf are the precise library functions.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void embed_sinusoid_kernel(
     float* __restrict__ out, const int* __restrict__ ids, const T* __restrict__ table,
-    float scale, const int* __restrict__ positions, const float* __restrict__ freqs,
+    float scale, const int* __restrict__ positions, const double* __restrict__ freqs,
     int S, int C) {
   const int t = blockIdx.x;
   const T* row = table + (size_t)ids[t] * C;
-  const float p = (float)positions[t];
+  const double p = (double)positions[t];
+  constexpr double kTwoPi = 6.283185307179586476925;
   for (int c = threadIdx.x; c < C; c += kBlock) {
-    const float ang = p * freqs[c >> 1];
+    double a = p * freqs[c >> 1];
+    a -= kTwoPi * floor(a / kTwoPi);
+    const float ang = (float)a;
     const float x = ldf(row + c) * scale + ((c & 1) ? cosf(ang) : sinf(ang));
     for (int s = 0; s < S; ++s) out[((size_t)t * S + s) * C + c] = x;
   }
@@ -148,7 +152,8 @@ void embed_sinusoid(torch::Tensor out, torch::Tensor ids, torch::Tensor table,
   check_f32(out, "out");
   check_i32(ids, "ids");
   check_i32(positions, "positions");
-  check_f32(freqs, "freqs");
+  TORCH_CHECK(freqs.scalar_type() == torch::kFloat64 && freqs.is_contiguous() &&
+              freqs.is_cuda(), "freqs must be a contiguous float64 GPU tensor");
   TORCH_CHECK(table.is_cuda() && table.is_contiguous() && table.dim() == 2 &&
               out.dim() == 3);
   const int T = out.size(0), S = out.size(1), C = out.size(2);
@@ -159,7 +164,7 @@ void embed_sinusoid(torch::Tensor out, torch::Tensor ids, torch::Tensor table,
     hipLaunchKernelGGL((embed_sinusoid_kernel<act_t>), dim3(T), dim3(kBlock), 0,
                        SEQ_STREAM(), (float*)out.data_ptr(), (const int*)ids.data_ptr(),
                        (const act_t*)table.data_ptr(), (float)scale,
-                       (const int*)positions.data_ptr(), (const float*)freqs.data_ptr(),
+                       (const int*)positions.data_ptr(), (const double*)freqs.data_ptr(),
                        S, C);
   });
   SEQ_CHECK_LAUNCH();

@@ -112,8 +112,9 @@ class VigonexLayer(nn.Module):
 
 
 def sinusoid_frequencies(width: int, base: float = 10000.0) -> torch.Tensor:
+    """float64 [ceil(width / 2)]: base^(-2 i / width)."""
     i = torch.arange((width + 1) // 2, dtype=torch.float64)
-    return (float(base) ** (-2.0 * i / width)).to(torch.float32)
+    return float(base) ** (-2.0 * i / width)
 
 
 class VigonexForCausalLM(nn.Module):

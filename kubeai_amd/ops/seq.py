@@ -792,15 +792,16 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
 def embed_sinusoid(ids, table, scale: float, positions, freqs, copies: int = 1):
     """fp32 [T, copies, C], every copy table[ids] * scale plus a position
     vector whose column c is sin (c even) or cos (c odd) of
-    position * freqs[c // 2] (fp32 angle). table [V, C] in the serving dtype,
-    freqs fp32 [ceil(C / 2)]."""
+    position * freqs[c // 2]. table [V, C] in the serving dtype, freqs
+    float64 [ceil(C / 2)]: the angle is formed in double and reduced to one
+    turn before the fp32 sine and cosine."""
     T, C = ids.shape[0], table.shape[1]
     if table.is_cuda:
         _require_ext()
         out = torch.empty((T, copies, C), dtype=torch.float32, device=table.device)
         _C.embed_sinusoid(out, ids, table, scale, positions, freqs)
         return out
-    ang = positions.float().unsqueeze(-1) * freqs  # [T, ceil(C/2)]
+    ang = torch.remainder(positions.double().unsqueeze(-1) * freqs, 2.0 * math.pi).float()
     pe = torch.stack([torch.sin(ang), torch.cos(ang)], dim=-1).reshape(T, -1)[:, :C]
     x = table[ids.long()].float() * scale + pe
     return x.unsqueeze(1).repeat(1, copies, 1)

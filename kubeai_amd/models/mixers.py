@@ -607,13 +607,17 @@ class RoutedGatedMoE(nn.Module):
     experts a token did not choose) folded into the activation, so the
     weighted sum happens inside the second GEMM's fp32 accumulation and the
     step has no data-dependent shapes. Large steps gather each expert's
-    tokens and run its slice."""
+    tokens and run its slice.
+
+    extra_out > 0 appends that many rows (with a bias) to the stacked input
+    matrix for a projection of the same input that the caller owns (a
+    residual gate); forward then returns (output, that projection)."""
 
     DENSE_MAX_TOKENS = 256
 
     def __init__(self, width, experts, top, ff, correction=True, act_alpha=1.0,
                  act_limit=0.0, up_shift=0.0, weight_scale=1.0, shared_ff=0,
-                 shared_limit=0.0, shared_gate=False):
+                 shared_limit=0.0, shared_gate=False, extra_out=0):
         super().__init__()
         self.experts, self.top, self.ff = experts, top, ff
         self.act = dict(alpha=float(act_alpha), limit=float(act_limit or 0.0),
@@ -628,7 +632,9 @@ class RoutedGatedMoE(nn.Module):
             requires_grad=False)
         nn.init.normal_(self.router, std=width ** -0.5)
         self.correction = _f32(experts) if correction else None
-        self.gate_up = Proj(width, experts * 2 * ff + 2 * self.shared_ff)
+        self.extra_out = int(extra_out or 0)
+        n_in = experts * 2 * ff + 2 * self.shared_ff + self.extra_out
+        self.gate_up = BiasProj(width, n_in) if self.extra_out else Proj(width, n_in)
         self.down = Proj(experts * ff + self.shared_ff, width)
 
     def forward(self, h):
@@ -639,15 +645,17 @@ class RoutedGatedMoE(nn.Module):
         dense, w, idx = sops.router_scores_topk(
             logits[:, :E] if self.shared_gate else logits, self.top, self.correction,
             self.weight_scale)
+        at = E * 2 * ff + 2 * sff  # where the caller's extra projection starts
         if T <= self.DENSE_MAX_TOKENS:
             gu = self.gate_up(h)
             a = torch.empty((T, E * ff + sff), dtype=h.dtype, device=h.device)
             sops.glu_weighted(gu[:, : E * 2 * ff], dense, ff, out=a[:, : E * ff],
                               **self.act)
             if sff:
-                sops.glu_weighted(gu[:, E * 2 * ff :], sg, sff, w_sigmoid=True,
+                sops.glu_weighted(gu[:, E * 2 * ff : at], sg, sff, w_sigmoid=True,
                                   out=a[:, E * ff :], **self.shared_act)
-            return self.down(a)
+            y = self.down(a)
+            return (y, gu[:, at:]) if self.extra_out else y
         out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
         flat = idx.flatten().long()
         order = torch.argsort(flat, stable=True)
@@ -666,25 +674,36 @@ class RoutedGatedMoE(nn.Module):
             y = F.linear(a, self.down.weight[:, e * ff : (e + 1) * ff])
             out.index_add_(0, rows, y.float())
             s += n
-        if sff:
-            gu = F.linear(h, self.gate_up.weight[E * 2 * ff :])
-            a = sops.glu_weighted(gu, sg, sff, w_sigmoid=True, **self.shared_act)
-            out.add_(F.linear(a, self.down.weight[:, E * ff :]))
-        return out
+        extra = None
+        if sff or self.extra_out:
+            # the shared expert's rows and the caller's are one product
+            bias = self.gate_up.bias[E * 2 * ff :] if self.extra_out else None
+            gu = F.linear(h, self.gate_up.weight[E * 2 * ff :], bias)
+            if sff:
+                a = sops.glu_weighted(gu[:, : 2 * sff], sg, sff, w_sigmoid=True,
+                                      **self.shared_act)
+                out.add_(F.linear(a, self.down.weight[:, E * ff :]))
+            extra = gu[:, 2 * sff :]
+        return (out, extra) if self.extra_out else out
 
 
 class SiluGatedMLP(nn.Module):
     """Dense gated feed-forward: down(silu(gate h) * (up h)); the gate and up
-    matrices are one stacked [2 ff, width] product."""
+    matrices are one stacked [2 ff, width] product. extra_out > 0 appends
+    that many rows (with a bias) for a projection of the same input that the
+    caller owns; forward then returns (output, that projection)."""
 
-    def __init__(self, width: int, ff: int):
+    def __init__(self, width: int, ff: int, extra_out: int = 0):
         super().__init__()
-        self.ff = ff
-        self.gate_up = Proj(width, 2 * ff)
+        self.ff, self.extra_out = ff, int(extra_out or 0)
+        n_in = 2 * ff + self.extra_out
+        self.gate_up = BiasProj(width, n_in) if self.extra_out else Proj(width, n_in)
         self.down = Proj(ff, width)
 
     def forward(self, h):
-        return self.down(sops.glu_weighted(self.gate_up(h), None, self.ff))
+        gu = self.gate_up(h)
+        y = self.down(sops.glu_weighted(gu[:, : 2 * self.ff], None, self.ff))
+        return (y, gu[:, 2 * self.ff :]) if self.extra_out else y
 
 
 class BiasProj(nn.Module):

@@ -65,7 +65,7 @@ def build_mlp(mlp: dict | None, width: int):
         return None
     kind = mlp.get("kind")
     if kind == "dense":
-        return SiluGatedMLP(width, int(mlp["ff"]))
+        return SiluGatedMLP(width, int(mlp["ff"]), extra_out=width)
     if kind == "moe":
         shared = mlp.get("shared") or {}
         return RoutedGatedMoE(
@@ -75,15 +75,17 @@ def build_mlp(mlp: dict | None, width: int):
             weight_scale=float(mlp["router"].get("scale", 1.0)),
             shared_ff=int(shared.get("ff", 0)),
             shared_limit=float(shared.get("limit") or 0.0), shared_gate=True,
+            extra_out=width,
         )
     raise ValueError(f"unknown feed-forward kind {kind!r}")
 
 
 class HyperConnection(nn.Module):
     """Read weights, write weights and the stream-to-stream matrix of one
-    sublayer, with its input norm and residual gate."""
+    sublayer, with its input norm and residual gate (own_gate=False: the
+    sublayer computes the gate's projection inside its own input product)."""
 
-    def __init__(self, width: int, streams: int):
+    def __init__(self, width: int, streams: int, own_gate: bool = True):
         super().__init__()
         self.norm = _f32(width)
         nn.init.ones_(self.norm)
@@ -93,7 +95,7 @@ class HyperConnection(nn.Module):
         nn.init.constant_(self.read, 1.0 / streams)
         nn.init.ones_(self.write)
         self.mix.data.copy_(torch.eye(streams))
-        self.gate = BiasProj(width, width)
+        self.gate = BiasProj(width, width) if own_gate else None
 
 
 class VigonexLayer(nn.Module):
@@ -102,7 +104,9 @@ class VigonexLayer(nn.Module):
         self.mixer = build_mixer(spec, width, eps)
         self.mlp = build_mlp(spec.mlp, width)
         self.hc1 = HyperConnection(width, streams)
-        self.hc2 = HyperConnection(width, streams) if self.mlp is not None else None
+        # the feed-forward's gate reads the feed-forward's input: one product
+        self.hc2 = (HyperConnection(width, streams, own_gate=False)
+                    if self.mlp is not None else None)
         self.shift = _f32(1, width)
 
     def state_spec(self):
@@ -194,8 +198,8 @@ class VigonexForCausalLM(nn.Module):
             y = layer.mixer(hin, fb, state, self.kv_caches[i])
             if layer.mlp is not None:
                 h = read(layer.hc2)
-                hc, gate = layer.hc2, layer.hc2.gate(h)
-                y = layer.mlp(h)
+                hc = layer.hc2
+                y, gate = layer.mlp(h)
             if self.capture_layers is not None:
                 self.capture_layers.append(self._streams_after(X, y, gate, hc))
         return sops.hyper_mix_rmsnorm(
@@ -251,8 +255,9 @@ class VigonexForCausalLM(nn.Module):
                     hc.read.data.fill_(1.0)
                     hc.write.data.fill_(1.0)
                     hc.mix.data.fill_(1.0)
-                put(hc.gate.weight, get(f"{p}rg{q}"))
-                put(hc.gate.bias, get(f"{p}rg{q}.b"))
+                if hc.gate is not None:
+                    put(hc.gate.weight, get(f"{p}rg{q}"))
+                    put(hc.gate.bias, get(f"{p}rg{q}.b"))
             m, q = layer.mixer, p + "mix."
             if isinstance(m, DifferentialAttention):
                 order = m.query_row_order()
@@ -277,8 +282,14 @@ class VigonexForCausalLM(nn.Module):
             f, q = layer.mlp, p + "mlp."
             if f is None:
                 continue
+            rg, rg_b = get(p + "rg2"), get(p + "rg2.b")
+
+            def with_gate_bias(n_rows):
+                return torch.cat([torch.zeros(n_rows, dtype=rg_b.dtype), rg_b])
+
             if isinstance(f, SiluGatedMLP):
-                put(f.gate_up.weight, torch.cat([get(q + "gate"), get(q + "up")]))
+                put(f.gate_up.weight, torch.cat([get(q + "gate"), get(q + "up"), rg]))
+                put(f.gate_up.bias, with_gate_bias(2 * f.ff))
                 put(f.down.weight, get(q + "down"))
             else:
                 names = [f"{q}e{e}." for e in range(f.experts)]
@@ -287,7 +298,8 @@ class VigonexForCausalLM(nn.Module):
                     names.append(q + "shared.")
                     router.append(get(q + "shared.sg").reshape(1, -1))
                 put(f.gate_up.weight, torch.cat(
-                    [get(n + part) for n in names for part in ("gate", "up")]))
+                    [get(n + part) for n in names for part in ("gate", "up")] + [rg]))
+                put(f.gate_up.bias, with_gate_bias(f.experts * 2 * f.ff + 2 * f.shared_ff))
                 put(f.down.weight, torch.cat([get(n + "down") for n in names], dim=1))
                 put(f.router, torch.cat(router))
         missing = set(W) - used

@@ -882,7 +882,7 @@ def vigonex_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 
     moe = {"kind": "moe", "expert": {"ff": ff_exp, "limit": 7.0},
            "router": {"experts": experts, "top": top, "scale": 1.0},
            "shared": {"ff": ff_exp, "limit": 7.0}}
-    att = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": head_dim, "diff": 0.3,
+    att = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": head_dim, "diff": 0.2,
            "scale": dim ** -0.5, "softcap": 30.0, "q_temp": {"coef": 0.1, "every": 1024}}
     ddim = min(64, head_dim)
     delta = {"heads": max(1, width // ddim), "dim": ddim, "lowrank": max(16, width // 32)}

@@ -198,11 +198,11 @@ def test_token_shift_carries_the_previous_token(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("coef,every", [(0.5, 3), (0.3, 64), (1.0, 1), (0.0, 5)])
+@pytest.mark.parametrize("coef,every", [(0.5, 3), (0.25, 48), (1.0, 1), (0.0, 5)])
 def test_query_temperature_and_cache_rows(device, coef, every):
     g = torch.Generator().manual_seed(every)
     H, G, Gv, D, Dv, bs = 4, 4, 2, 6, 10, 4
-    pos = [0, 1, 2, 3, 5, 62, 63, 64, 127, 128, 191]  # both sides of every step of the floor
+    pos = [0, 1, 2, 3, 5, 46, 47, 48, 94, 95, 96, 143]  # both sides of every step of the floor
     T = len(pos)
     q, k, v = (torch.randn(T, n, d, generator=g) for n, d in ((H, D), (G, D), (Gv, Dv)))
     kc, vc = torch.zeros(60, G, bs, D, device=device), torch.zeros(60, Gv, bs, Dv, device=device)
@@ -212,7 +212,7 @@ def test_query_temperature_and_cache_rows(device, coef, every):
     sops.scale_q_and_cache(qd, k.to(device), v.to(device),
                            torch.tensor(pos, dtype=torch.int32, device=device), coef, every,
                            kc, vc, slots.to(device))
-    temp = oracle.query_temperature(192, {"coef": coef, "every": every} if coef else None)
+    temp = oracle.query_temperature(144, {"coef": coef, "every": every} if coef else None)
     assert np.abs(npy(qd) - npy(q) * temp[pos][:, None, None]).max() < 1e-5
     for i, p in enumerate(pos):
         s = p + 7
@@ -405,17 +405,17 @@ def test_delta_rule_removes_what_a_key_held(device):
 @pytest.mark.parametrize("device", DEVICES)
 def test_router_weights_scale_and_clamped_activation(device):
     z = torch.tensor([[0.1, 2.0, -1.0, 2.0, 0.5], [3.0, -3.0, 0.0, 1.0, 2.9]])
-    dense, w, idx = sops.router_scores_topk(z.to(device), 2, None, 1.5)
+    dense, w, idx = sops.router_scores_topk(z.to(device), 2, None, 1.7)
     s = torch.softmax(z, -1)
     assert idx.cpu().tolist() == [[1, 3], [0, 4]]  # ties: the lower index first
-    assert np.allclose(npy(w), npy(torch.gather(s, 1, idx.cpu().long()) * 1.5), atol=1e-6)
+    assert np.allclose(npy(w), npy(torch.gather(s, 1, idx.cpu().long()) * 1.7), atol=1e-6)
     assert np.allclose(npy(dense).sum(-1), npy(w).sum(-1), atol=1e-6)
     g = torch.Generator().manual_seed(5)
     gu = 3.0 * torch.randn(7, 2 * 3 * 8, generator=g)  # three experts of 8
     rw = torch.rand(7, 3, generator=g)
-    got = sops.glu_weighted(gu.to(device), rw.to(device), 8, alpha=1.702, limit=2.0, up_shift=1.0)
+    got = sops.glu_weighted(gu.to(device), rw.to(device), 8, alpha=1.702, limit=1.8, up_shift=1.0)
     a = npy(gu).reshape(7, 3, 2, 8)
-    gate, up = np.minimum(a[:, :, 0], 2.0), np.clip(a[:, :, 1], -2.0, 2.0)
+    gate, up = np.minimum(a[:, :, 0], 1.8), np.clip(a[:, :, 1], -1.8, 1.8)
     want = gate * oracle.sigmoid(1.702 * gate) * (up + 1.0) * npy(rw)[:, :, None]
     assert np.abs(npy(got) - want.reshape(7, 24)).max() < 1e-5
     # no weight, no clamp: plain silu(gate) * up; sigmoid of the weight column
@@ -761,7 +761,7 @@ def test_kernel_activation_embedding_join(dtype):
     for group, n, pad in ((8, 3, 0), (96, 12, 0), (5, 2, 0), (64, 4, 16)):
         gu = (2.0 * torch.randn(33, n * 2 * group + pad, generator=g)).to(dtype)[:, : n * 2 * group]
         rw = torch.rand(33, n, generator=g)
-        for kw in (dict(alpha=1.702, limit=1.5, up_shift=1.0), dict(), dict(w_sigmoid=True)):
+        for kw in (dict(alpha=1.702, limit=1.25, up_shift=1.0), dict(), dict(w_sigmoid=True)):
             _close(sops.glu_weighted(gu.cuda(), rw.cuda(), group, **kw),
                    sops.glu_weighted(gu, rw, group, **kw), dtype)
         _close(sops.glu_weighted(gu.cuda(), None, group), sops.glu_weighted(gu, None, group), dtype)
@@ -770,8 +770,8 @@ def test_kernel_activation_embedding_join(dtype):
     ids = torch.randint(0, 50, (40,), generator=g, dtype=torch.int32)
     pos = torch.randint(0, 3000, (40,), generator=g, dtype=torch.int32)
     f = sinusoid_frequencies(200)
-    got = sops.embed_sinusoid(ids.cuda(), table.cuda(), 3.0, pos.cuda(), f.cuda(), 2)
-    want = sops.embed_sinusoid(ids, table, 3.0, pos, f, 2)
+    got = sops.embed_sinusoid(ids.cuda(), table.cuda(), 2.5, pos.cuda(), f.cuda(), 2)
+    want = sops.embed_sinusoid(ids, table, 2.5, pos, f, 2)
     assert float((got.cpu() - want).abs().max()) < (1e-5 if dtype == torch.float32 else 0.1)
     att_ = torch.randn(21, 2, 2, 3, 40, generator=g).to(dtype)
     out = torch.zeros(21, 6, 40, dtype=dtype)
